@@ -218,7 +218,7 @@ constexpr int kMergeThreads = 256;
 __global__ __launch_bounds__(kMergeThreads) void attn_decode_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ positions,
     const int* __restrict__ token_list, bf16_t* __restrict__ out, int window_kind, int window, int nh, int hd,
-    int max_splits, int sink) {
+    int max_splits, int sink, const float* __restrict__ sink_vals) {
   __shared__ float red_s[kMergeThreads / kWave];
   __shared__ f32x4 o_s[kMergeThreads];
   __shared__ float l_s[kMergeThreads];
@@ -269,7 +269,7 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_merge_kernel(
     o += o_s[x * ncol + col];
     L += l_s[x * ncol + col];
   }
-  if (sink && M > -INFINITY) L += expf(-M);   // a key of score 0 without a value: one more term in the denominator
+  if (sink && M > -INFINITY) L += expf((sink_vals ? sink_vals[h] : 0.f) - M);   // a key of score 0 without a value: one more term in the denominator
   unsigned short b[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) b[i] = runs_wanted > max_splits ? (unsigned short)0x7fc0 : f32_to_bf16(L > 0.f ? o[i] / L : 0.f).bits;
@@ -284,7 +284,7 @@ static int launch_decode(const void* q, const void* k_cache, const void* v_cache
                          const int* entry_of_token, const int* positions, const int* token_list, float* part_o,
                          float* part_ml, void* out, int window_kind, int window, float scale, int n_list, int nh,
                          int nkv, int page_size, int max_blocks, int num_pages, int max_splits, float softcap, int sink,
-                         hipStream_t stream) {
+                         const float* sink_vals, hipStream_t stream) {
   const int G = nh / nkv;
   dim3 grid(nkv * ((G + 15) / 16), n_list, max_splits), block(kDecWaves * kWave);
   attn_decode_kernel<HD><<<grid, block, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
@@ -294,7 +294,7 @@ static int launch_decode(const void* q, const void* k_cache, const void* v_cache
   SHARPI_CHECK_LAUNCH();
   dim3 mgrid(n_list, nh), mblock(kMergeThreads);
   attn_decode_merge_kernel<<<mgrid, mblock, 0, stream>>>(part_o, part_ml, positions, token_list, (bf16_t*)out,
-                                                         window_kind, window, nh, HD, max_splits, sink);
+                                                         window_kind, window, nh, HD, max_splits, sink, sink_vals);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
@@ -306,13 +306,14 @@ static int launch_decode(const void* q, const void* k_cache, const void* v_cache
 // runs of 256 keys (runs are aligned to absolute positions, so a window that starts inside a run
 // takes one more than its length suggests); ((context - 1) >> 4) / 16 + 1 covers every window of a
 // context.  A token whose runs exceed max_splits gets a row of NaN.  softcap > 0: scores become
-// softcap * tanh(score / softcap); sink: the denominator holds one more term exp(0).
+// softcap * tanh(score / softcap); sink: the denominator holds one more term exp(0), or, with sink_vals
+// (float [nh]), exp(sink_vals[head]): a learned score per head that is not scaled.
 SHARPI_EXPORT int sharpi_attention_decode(const void* q, const void* k_cache, const void* v_cache,
                                           const int* block_table, const int* entry_of_token, const int* positions,
                                           const int* token_list, float* part_o, float* part_ml, void* out,
                                           int window_kind, int window, float scale, int n_list, int nh, int nkv,
                                           int hd, int page_size, int max_blocks, int num_pages, int max_splits,
-                                          float softcap, int sink, hipStream_t stream) {
+                                          float softcap, int sink, const float* sink_vals, hipStream_t stream) {
   if (n_list <= 0) return SHARPI_OK;
   if (nh <= 0 || nkv <= 0 || nh % nkv != 0 || nh > 65535 || n_list > 65535) return SHARPI_ERR_ARG;
   if (page_size <= 0 || page_size % 16 != 0 || max_blocks <= 0 || num_pages <= 0 || max_splits <= 0 || max_splits > 65535) return SHARPI_ERR_ARG;
@@ -322,7 +323,7 @@ SHARPI_EXPORT int sharpi_attention_decode(const void* q, const void* k_cache, co
   if (hd == HDV)                                                                                                  \
     return launch_decode<HDV>(q, k_cache, v_cache, block_table, entry_of_token, positions, token_list, part_o,    \
                               part_ml, out, window_kind, window, scale, n_list, nh, nkv, page_size, max_blocks,   \
-                              num_pages, max_splits, softcap, sink, stream);
+                              num_pages, max_splits, softcap, sink, sink_vals, stream);
   SHARPI_DECODE_HEAD_SIZES(DEC)
 #undef DEC
   return SHARPI_ERR_ARG;  // other head sizes go to the generic kernel
@@ -382,5 +383,5 @@ int sharpi_attention_decode_noalloc(const void* q, const void* k_cache, const vo
   float* part_ml = ws + runs * (unsigned long long)hd;   // hd is a multiple of 32: stays 16-byte aligned
   return sharpi_attention_decode(q, k_cache, v_cache, block_table, entry_of_token, positions, token_list, part_o,
                                  part_ml, out, window_kind, window, scale, n_list, nh, nkv, hd, page_size, max_blocks,
-                                 num_pages, max_splits, 0.f, 0, stream);
+                                 num_pages, max_splits, 0.f, 0, nullptr, stream);
 }

@@ -7,7 +7,8 @@
 // the order of every sum depends on (start, p) alone: not on how the tokens were batched.
 // Values may have another width than keys (vd): q and keys are hd wide, values and the output vd.
 // softcap > 0 bends every score to softcap * tanh(score / softcap) before the mask; with `sink` the
-// softmax's denominator holds one more term, exp(0): a key of score 0 that has no value.
+// softmax's denominator holds one more term, exp(0): a key of score 0 that has no value (or, with
+// sink_vals, exp(sink_vals[head]): a learned score per head, not scaled).
 #include "common.h"
 
 constexpr int kAttnWaves = 4;
@@ -18,7 +19,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_table, const int* __restrict__ entry_of_token,
     const int* __restrict__ positions, T* __restrict__ out, int window_kind, int window, float scale, int nh,
-    int nkv, int hd, int vd, int page_size, int max_blocks, int num_pages, float softcap, int sink) {
+    int nkv, int hd, int vd, int page_size, int max_blocks, int num_pages, float softcap, int sink, const float* __restrict__ sink_vals) {
   __shared__ float qs[kAttnMaxHd];
   __shared__ float pw[kAttnWaves][kWave];
   __shared__ int vrow[kAttnWaves][kWave];
@@ -116,7 +117,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
     f[i] = m_s[i] > -INFINITY ? expf(m_s[i] - M) : 0.f;
     L += l_s[i] * f[i];
   }
-  if (sink) L += expf(-M);   // (every query sees at least its own key, so M is finite)
+  if (sink) L += expf((sink_vals ? sink_vals[h] : 0.f) - M);   // (every query sees at least its own key, so M is finite)
   T* orow = out + ((size_t)t * nh + h) * vd;
   for (int d = threadIdx.x; d < vd; d += blockDim.x) {
     float o = 0.f;
@@ -129,7 +130,7 @@ SHARPI_EXPORT int sharpi_attention_generic(const void* q, const void* k_cache, c
                                            const int* block_table, const int* entry_of_token,
                                            const int* positions, void* out, int window_kind, int window,
                                            float scale, int n_tokens, int nh, int nkv, int hd, int vd, int page_size,
-                                           int max_blocks, int num_pages, float softcap, int sink, hipStream_t stream) {
+                                           int max_blocks, int num_pages, float softcap, int sink, const float* sink_vals, hipStream_t stream) {
   if (n_tokens <= 0) return SHARPI_OK;
   if (hd <= 0 || hd > kAttnMaxHd || vd <= 0 || vd > kAttnMaxHd || nh <= 0 || nkv <= 0 || nh % nkv != 0 || nh > 65535) return SHARPI_ERR_ARG;
   if (page_size <= 0 || max_blocks <= 0 || num_pages <= 0) return SHARPI_ERR_ARG;
@@ -138,11 +139,11 @@ SHARPI_EXPORT int sharpi_attention_generic(const void* q, const void* k_cache, c
   if (dtype == DT_F32)
     attn_generic_kernel<float><<<grid, block, 0, stream>>>(
         (const float*)q, (const float*)k_cache, (const float*)v_cache, block_table, entry_of_token, positions,
-        (float*)out, window_kind, window, scale, nh, nkv, hd, vd, page_size, max_blocks, num_pages, softcap, sink);
+        (float*)out, window_kind, window, scale, nh, nkv, hd, vd, page_size, max_blocks, num_pages, softcap, sink, sink_vals);
   else if (dtype == DT_BF16)
     attn_generic_kernel<bf16_t><<<grid, block, 0, stream>>>(
         (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, entry_of_token, positions,
-        (bf16_t*)out, window_kind, window, scale, nh, nkv, hd, vd, page_size, max_blocks, num_pages, softcap, sink);
+        (bf16_t*)out, window_kind, window, scale, nh, nkv, hd, vd, page_size, max_blocks, num_pages, softcap, sink, sink_vals);
   else
     return SHARPI_ERR_ARG;
   SHARPI_CHECK_LAUNCH();

@@ -74,7 +74,7 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? (kQT == 1 ? 3 : 2) : 
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, const int* __restrict__ positions, const int* __restrict__ tiles,
     bf16_t* __restrict__ out, int window_kind, int window, float scale, int nh, int nkv, int page_size,
-    int max_blocks, int num_pages, float softcap, int sink) {
+    int max_blocks, int num_pages, float softcap, int sink, const float* __restrict__ sink_vals) {
   constexpr int kWaveTokens = 16 * kQT;
   constexpr int NJ = HD / 32;
   constexpr int ND = HD / 16;
@@ -371,7 +371,8 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? (kQT == 1 ? 3 : 2) : 
     L += __shfl_xor(L, 16, kWave);
     L += __shfl_xor(L, 32, kWave);
     if (!qok[c]) continue;
-    if (sink) L += __builtin_amdgcn_exp2f(-m[c]);   // a key of score 0 without a value: 2^(0 - reference) more
+    // a key of score 0 (or of the head's learned score) without a value: 2^(score log2 e - reference) more
+    if (sink) L += __builtin_amdgcn_exp2f((sink_vals ? sink_vals[h] * 1.4426950408889634f : 0.f) - m[c]);
     const float inv = L > 0.f ? 1.0f / L : 0.f;
     bf16_t* orow = out + ((size_t)(tok0 + wrow0 + c * 16 + r) * nh + h) * HD;
 #pragma unroll
@@ -390,12 +391,14 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? (kQT == 1 ? 3 : 2) : 
 // tiles int32 [n_tiles, 3] = (entry, first token, rows <= tile_tokens), tokens of a tile consecutive
 // in one entry; tile_tokens 128 or 64 (what the caller cut the tiles to: no tile may hold more);
 // out [T, nh, hd] bf16 (rows of the listed tiles).  softcap > 0: scores become softcap * tanh(score /
-// softcap); sink: the denominator holds one more term exp(0).
+// softcap); sink: the denominator holds one more term exp(0), or, with sink_vals (float [nh]),
+// exp(sink_vals[head]): a learned score per head that is not scaled.
 SHARPI_EXPORT int sharpi_attention_prefill(const void* q, const void* k_cache, const void* v_cache,
                                            const int* block_table, const int* positions, const int* tiles,
                                            void* out, int n_tiles, int tile_tokens, int window_kind, int window,
                                            float scale, int nh, int nkv, int hd, int page_size, int max_blocks,
-                                           int num_pages, float softcap, int sink, hipStream_t stream) {
+                                           int num_pages, float softcap, int sink, const float* sink_vals,
+                                           hipStream_t stream) {
   if (n_tiles <= 0) return SHARPI_OK;
   if (nh <= 0 || nkv <= 0 || nh % nkv != 0 || n_tiles > 65535) return SHARPI_ERR_ARG;
   if (tile_tokens != kTileTokens && tile_tokens != kTileTokens / 2) return SHARPI_ERR_ARG;
@@ -406,7 +409,7 @@ SHARPI_EXPORT int sharpi_attention_prefill(const void* q, const void* k_cache, c
   attn_prefill_kernel<HDV, QTV><<<grid, block, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache,               \
                                                            (const bf16_t*)v_cache, block_table, positions, tiles,  \
                                                            (bf16_t*)out, window_kind, window, scale, nh, nkv,      \
-                                                           page_size, max_blocks, num_pages, softcap, sink)
+                                                           page_size, max_blocks, num_pages, softcap, sink, sink_vals)
 #define PRE(HDV)                                  \
   if (hd == HDV) {                                \
     if (tile_tokens == kTileTokens) PRE_QT(HDV, 2); \

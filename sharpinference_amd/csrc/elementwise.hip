@@ -262,23 +262,28 @@ SHARPI_EXPORT int sharpi_add_rmsnorm(float* h, const void* delta, int delta_dtyp
 
 // ---------------------------------------------------------------------------
 // The gated unit on a fused [M, 2*I] buffer (gate columns first, up columns second):
-//   out[m, i] = act(s_m * g) * (s_m * u),  s_m = scale ? scale[m] : 1,  act as common.h codes it
+//   out[m, i] = act(s_m * g) * (s_m * u),  s_m = scale ? scale[m] : 1,  act as common.h codes it;
+//   bias (float [2*I], optional) is added to g and u first, in float
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void silu_mul_kernel(const T* __restrict__ gu, const float* __restrict__ scale,
-                                T* __restrict__ out, int inter, int act) {
+                                T* __restrict__ out, int inter, int act, const float* __restrict__ bias) {
   const int m = blockIdx.x;
   const int i = blockIdx.y * blockDim.x + threadIdx.x;
   if (i >= inter) return;
   const T* row = gu + (size_t)m * 2 * inter;
-  const float g = to_f32<T>(row[i]);
-  const float u = to_f32<T>(row[inter + i]);
+  float g = to_f32<T>(row[i]);
+  float u = to_f32<T>(row[inter + i]);
+  if (bias) {
+    g += bias[i];
+    u += bias[inter + i];
+  }
   out[(size_t)m * inter + i] = from_f32<T>(gated_f32(act, g, u, scale ? scale[m] : 1.0f, scale != nullptr));
 }
 
 template <typename T>
 __global__ void silu_mul_vec_kernel(const T* __restrict__ gu, const float* __restrict__ scale,
-                                    T* __restrict__ out, int inter, int act) {
+                                    T* __restrict__ out, int inter, int act, const float* __restrict__ bias) {
   const int m = blockIdx.x;
   const int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
   if (i >= inter) return;
@@ -286,6 +291,13 @@ __global__ void silu_mul_vec_kernel(const T* __restrict__ gu, const float* __res
   float g[8], u[8], o[8];
   load8(row + i, g);
   load8(row + inter + i, u);
+  if (bias) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      g[j] += bias[i + j];
+      u[j] += bias[inter + i + j];
+    }
+  }
   const float s = scale ? scale[m] : 1.0f;
 #pragma unroll
   for (int j = 0; j < 8; ++j) o[j] = gated_f32(act, g[j], u[j], s, scale != nullptr);
@@ -293,7 +305,7 @@ __global__ void silu_mul_vec_kernel(const T* __restrict__ gu, const float* __res
 }
 
 SHARPI_EXPORT int sharpi_silu_mul(const void* gu, const float* scale, void* out, int dtype, int rows, int inter,
-                                  int act, hipStream_t stream) {
+                                  int act, const float* bias, hipStream_t stream) {
   if (rows <= 0) return SHARPI_OK;
   if (inter <= 0 || ceil_div(inter, 256) > 65535 || !act_known(act)) return SHARPI_ERR_ARG;
   dim3 block(256), grid(rows, ceil_div(inter, 256));
@@ -301,13 +313,13 @@ SHARPI_EXPORT int sharpi_silu_mul(const void* gu, const float* scale, void* out,
   if ((inter & 7) == 0) {
     dim3 vgrid(rows, ceil_div(inter, 256 * 8));
     if (dtype == DT_F32)
-      silu_mul_vec_kernel<float><<<vgrid, block, 0, stream>>>((const float*)gu, scale, (float*)out, inter, act);
+      silu_mul_vec_kernel<float><<<vgrid, block, 0, stream>>>((const float*)gu, scale, (float*)out, inter, act, bias);
     else
-      silu_mul_vec_kernel<bf16_t><<<vgrid, block, 0, stream>>>((const bf16_t*)gu, scale, (bf16_t*)out, inter, act);
+      silu_mul_vec_kernel<bf16_t><<<vgrid, block, 0, stream>>>((const bf16_t*)gu, scale, (bf16_t*)out, inter, act, bias);
   } else if (dtype == DT_F32)
-    silu_mul_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, scale, (float*)out, inter, act);
+    silu_mul_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, scale, (float*)out, inter, act, bias);
   else
-    silu_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, scale, (bf16_t*)out, inter, act);
+    silu_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, scale, (bf16_t*)out, inter, act, bias);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }

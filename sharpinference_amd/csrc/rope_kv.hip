@@ -21,14 +21,14 @@ __global__ void rope_kv_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
                                const int* __restrict__ positions, const float* __restrict__ inv_freq,
                                const float* __restrict__ bias,
                                int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale,
-                               int nh, int nkv, int hd, int vd, int page_size, int half_split, int rotary_dim) {
+                               int nh, int nkv, int hd, int vd, int page_size, int half_split, int rotary_dim,
+                               int row_stride) {
   const int t = blockIdx.x;
   const int head = blockIdx.y;            // 0..nh-1 q, nh..nh+nkv-1 k, then v
   const int lane = threadIdx.x;           // one wave
   const int half = hd >> 1;
-  const size_t row_width = (size_t)(nh + nkv) * hd + (size_t)nkv * vd;
   const size_t head_at = head < nh + nkv ? (size_t)head * hd : (size_t)(nh + nkv) * hd + (size_t)(head - nh - nkv) * vd;
-  const T* src = qkv + (size_t)t * row_width + head_at;
+  const T* src = qkv + (size_t)t * row_stride + head_at;
   const float* hb = bias ? bias + head_at : nullptr;
   const int pos = positions[t];
   const bool is_q = head < nh;
@@ -134,13 +134,13 @@ __global__ __launch_bounds__(256) void rope_kv_vec_kernel(
     const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
     const int* __restrict__ slot_mapping, const int* __restrict__ positions, const float* __restrict__ inv_freq,
     const float* __restrict__ bias, int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale,
-    int nh, int nkv, int hd, int page_size, int rotary_dim) {
+    int nh, int nkv, int hd, int page_size, int rotary_dim, int row_stride) {
   const int t = blockIdx.x;
   const int per_head = hd >> 3;                    // lanes per head: 4, 8, 16 or 32
   const int chunks = (nh + 2 * nkv) * per_head;
   const int pos = positions[t];
   const int slot = slot_mapping[t];
-  const T* src = qkv + (size_t)t * (nh + 2 * nkv) * hd;
+  const T* src = qkv + (size_t)t * row_stride;
   float post = 1.0f;
   if (temp_tuning) post = 1.0f + attn_scale * logf(floorf(((float)pos + 1.0f) / floor_scale) + 1.0f);
   // a thread's run within a head is the same in every turn of the loop (the block size is a multiple
@@ -218,7 +218,7 @@ SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, vo
                                  const int* slot_mapping, const int* positions, const float* inv_freq,
                                  const float* bias, int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale,
                                  int n_tokens, int nh, int nkv, int hd, int vd, int page_size, int pair_layout,
-                                 int rotary_dim, hipStream_t stream) {
+                                 int rotary_dim, int row_stride, hipStream_t stream) {
   if (n_tokens <= 0) return SHARPI_OK;
   // pair_layout: 0 = pairs (2i, 2i+1), 1 = pairs (i, i + rotary_dim/2); rotary_dim even, <= hd
   if (pair_layout < 0 || pair_layout > 1) return SHARPI_ERR_ARG;
@@ -226,10 +226,15 @@ SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, vo
   else if (rotary_dim <= 0 || (rotary_dim & 1) || rotary_dim > hd) return SHARPI_ERR_ARG;
   if (hd <= 0 || (hd & 1) || hd > 512 || vd <= 0 || nh <= 0 || nkv <= 0 || page_size <= 0) return SHARPI_ERR_ARG;
   if (nh + 2 * nkv > 65535) return SHARPI_ERR_ARG;
+  // rows of qkv may be wider than q, k and v (further columns behind them): row_stride elements a row, 0 = dense
+  const int row_width = (nh + nkv) * hd + nkv * vd;
+  if (row_stride == 0) row_stride = row_width;
+  if (row_stride < row_width) return SHARPI_ERR_ARG;
   if (temp_tuning && !(floor_scale > 0.f)) return SHARPI_ERR_ARG;
   dim3 grid(n_tokens, nh + 2 * nkv), block(kWave);
   if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;
-  if ((hd == 32 || hd == 64 || hd == 128 || hd == 256) && vd == hd && pair_layout == 0 && (rotary_dim & 7) == 0) {
+  if ((hd == 32 || hd == 64 || hd == 128 || hd == 256) && vd == hd && pair_layout == 0 && (rotary_dim & 7) == 0 &&
+      (row_stride & 7) == 0) {
     // a few tokens (decode): a token's heads over several blocks, for the compute units' sake;
     // many tokens: one block per token, which then computes its angles once for all heads
     const dim3 vgrid(n_tokens, n_tokens <= 64 ? ceil_div((nh + 2 * nkv) * (hd >> 3), 256) : 1);
@@ -237,12 +242,12 @@ SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, vo
       rope_kv_vec_kernel<float><<<vgrid, 256, 0, stream>>>((const float*)qkv, (float*)q_out, (float*)k_cache,
                                                              (float*)v_cache, slot_mapping, positions, inv_freq,
                                                              bias, qk_norm, eps, temp_tuning, floor_scale, attn_scale,
-                                                             nh, nkv, hd, page_size, rotary_dim);
+                                                             nh, nkv, hd, page_size, rotary_dim, row_stride);
     else
       rope_kv_vec_kernel<bf16_t><<<vgrid, 256, 0, stream>>>((const bf16_t*)qkv, (bf16_t*)q_out,
                                                               (bf16_t*)k_cache, (bf16_t*)v_cache, slot_mapping,
                                                               positions, inv_freq, bias, qk_norm, eps, temp_tuning,
-                                                              floor_scale, attn_scale, nh, nkv, hd, page_size, rotary_dim);
+                                                              floor_scale, attn_scale, nh, nkv, hd, page_size, rotary_dim, row_stride);
     SHARPI_CHECK_LAUNCH();
     return SHARPI_OK;
   }
@@ -250,12 +255,12 @@ SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, vo
     rope_kv_kernel<float><<<grid, block, 0, stream>>>((const float*)qkv, (float*)q_out, (float*)k_cache,
                                                      (float*)v_cache, slot_mapping, positions, inv_freq, bias, qk_norm,
                                                      eps, temp_tuning, floor_scale, attn_scale, nh, nkv, hd, vd,
-                                                     page_size, pair_layout, rotary_dim);
+                                                     page_size, pair_layout, rotary_dim, row_stride);
   else if (dtype == DT_BF16)
     rope_kv_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache,
                                                       (bf16_t*)v_cache, slot_mapping, positions, inv_freq, bias,
                                                       qk_norm, eps, temp_tuning, floor_scale, attn_scale, nh, nkv,
-                                                      hd, vd, page_size, pair_layout, rotary_dim);
+                                                      hd, vd, page_size, pair_layout, rotary_dim, row_stride);
   else
     return SHARPI_ERR_ARG;
   SHARPI_CHECK_LAUNCH();

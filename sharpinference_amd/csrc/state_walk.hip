@@ -1,0 +1,387 @@
+// Matrix-valued recurrent states with one scalar decay per (token, head), walked token by token.
+//
+// Per head a state S [dk, dv] (float) moves as S_t = a_t S_(t-1) + b_t k_t v_t^T and gives o_t = S_t^T q_t.
+// Two designs of mixer share the walk; they differ in where a_t and b_t come from and in what is done
+// with o_t:
+//   WALK_EXP_GATES  (a matrix memory with exponential gates): from pre-activations x_i, x_f of a token's
+//       head, i = cap tanh((x_i + bias_i) / cap), f = log_sigmoid(cap tanh((x_f + bias_f) / cap)), a running
+//       maximum m_t = max(f + m_(t-1), i) (m starts at 0), a_t = exp(f + m_(t-1) - m_t), b_t = exp(i - m_t);
+//       beside S a vector n_t = a_t n_(t-1) + b_t k_t; the output is o_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6).
+//   WALK_STATE_SPACE (a selective state space): dt = softplus(x_dt + bias_dt), a_t = exp(-exp(A_log) dt),
+//       b_t = dt; k and q are the state's input and output vectors, shared by the heads of a group; the
+//       output is o_t + D v_t.
+// Everything but the reading of q, k, v is float: the gates, their logarithms and exponentials, the
+// running maximum, the state, the sums.
+//
+// Work: a block (one wave) = (entry, head, 8 value columns).  Lane (g, j) keeps RPL = DKP / 8 rows
+// g RPL .. g RPL + RPL - 1 of column j in registers (DKP = dk rounded up to 32, 64, 128 or 256; rows
+// beyond dk stay zero).  Tokens are staged 16 at a time into LDS: q and k as floats in the order the
+// lanes read them, the 16 tokens' gates computed side by side (the running maximum by a scan over
+// the lanes whose order is fixed by the chunk), then the wave walks the 16 tokens.  A request's
+// state lies slice by slice, [heads, ceil(dv / 8), slice], a slice = RPL x 64 floats of S in the
+// lanes' order (row g RPL + r of column j at r 64 + 8 g + j), and, for the exponential gates, DKP
+// floats of n and the maximum m (each slice its own copy: the blocks of a head do not wait for
+// each other).
+#include "common.h"
+
+enum : int { WALK_EXP_GATES = 0, WALK_STATE_SPACE = 1 };
+constexpr int kWalkCols = 8;       // value columns of a block
+constexpr int kWalkChunk = 16;     // tokens staged at a time
+constexpr float kWalkFloor = 1e-6f;
+
+SHARPI_EXPORT int sharpi_state_walk_cols() { return kWalkCols; }
+
+// floats of a slice: S, then (exponential gates) n and 8 floats that begin with m
+static inline __host__ __device__ int walk_slice_floats(int dkp, int mode) {
+  return (dkp / 8) * 64 + (mode == WALK_EXP_GATES ? dkp + 8 : 0);
+}
+SHARPI_EXPORT int sharpi_state_walk_slice_floats(int dk, int mode) {
+  const int dkp = dk <= 32 ? 32 : dk <= 64 ? 64 : dk <= 128 ? 128 : 256;
+  return walk_slice_floats(dkp, mode);
+}
+
+__device__ __forceinline__ float softplus_f32(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+__device__ __forceinline__ float log_sigmoid_f32(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
+
+// where row `row` (= g RPL + r) of a staged q or k vector lies in LDS: four rows of a lane together,
+// the eight row groups side by side (a lane reads float4s, the wave 32 consecutive words)
+template <int RPL>
+__device__ __forceinline__ int staged_at(int row) {
+  const int g = row / RPL, r = row % RPL;
+  return ((r >> 2) * 8 + g) * 4 + (r & 3);
+}
+
+template <typename T, int RPL, int MODE>
+__global__ __launch_bounds__(kWave) void state_walk_kernel(
+    const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off, int heads_per_group,
+    const float* __restrict__ gates, int gate_stride, const float* __restrict__ p0, const float* __restrict__ p1,
+    const float* __restrict__ p2, float cap, float q_scale, float* __restrict__ state,
+    const int* __restrict__ state_slots, const int* __restrict__ cu_tokens, float* __restrict__ out, int nh, int dk,
+    int dv, int ncb) {
+  constexpr int DKP = RPL * 8;
+  __shared__ __attribute__((aligned(16))) float q_s[kWalkChunk][DKP];
+  __shared__ __attribute__((aligned(16))) float k_s[kWalkChunk][DKP];
+  __shared__ float v_s[kWalkChunk][kWalkCols];
+  __shared__ float a_s[kWalkChunk], b_s[kWalkChunk], e_s[kWalkChunk];
+  const int cb = blockIdx.x, h = blockIdx.y, e = blockIdx.z;
+  const int lane = threadIdx.x, g = lane >> 3, j = lane & 7;
+  const int t_first = cu_tokens[e], t_end = cu_tokens[e + 1];
+  if (t_end <= t_first) return;
+  const int slice = walk_slice_floats(DKP, MODE);
+  float* st = state + (((size_t)state_slots[e] * nh + h) * ncb + cb) * slice;
+  const int c = cb * kWalkCols + j;
+  const int qk_head = h / heads_per_group;
+
+  float S[RPL], n[RPL];
+#pragma unroll
+  for (int r = 0; r < RPL; ++r) S[r] = st[r * 64 + lane];
+  float m_run = 0.f;
+  if (MODE == WALK_EXP_GATES) {
+    const float4* nsrc = reinterpret_cast<const float4*>(st + RPL * 64);
+#pragma unroll
+    for (int r4 = 0; r4 < RPL / 4; ++r4) {
+      const float4 x = nsrc[r4 * 8 + g];
+      n[r4 * 4] = x.x; n[r4 * 4 + 1] = x.y; n[r4 * 4 + 2] = x.z; n[r4 * 4 + 3] = x.w;
+    }
+    m_run = st[RPL * 64 + DKP];
+  }
+  float par0 = 0.f, par1 = 0.f, par2 = 0.f;     // the head's constants
+  if (MODE == WALK_EXP_GATES) {
+    par0 = p0[h];
+    par1 = p1[h];
+  } else {
+    par0 = p0[h];                 // dt bias
+    par1 = -expf(p1[h]);          // -exp(A_log)
+    par2 = p2[h];                 // D
+  }
+
+  for (int t0 = t_first; t0 < t_end; t0 += kWalkChunk) {
+    const int nt = min(kWalkChunk, t_end - t0);
+    __syncthreads();
+    // stage q and k (floats, the lanes' order), v, and the tokens' gates
+    for (int idx = lane; idx < kWalkChunk * DKP; idx += kWave) {
+      const int tt = idx / DKP, row = idx % DKP;
+      float qv = 0.f, kv = 0.f;
+      if (tt < nt && row < dk) {
+        const T* base = proj + (size_t)(t0 + tt) * stride + (size_t)qk_head * dk + row;
+        qv = to_f32<T>(base[q_off]) * q_scale;
+        kv = to_f32<T>(base[k_off]);
+      }
+      const int at = staged_at<RPL>(row);
+      q_s[tt][at] = qv;
+      k_s[tt][at] = kv;
+    }
+    for (int idx = lane; idx < kWalkChunk * kWalkCols; idx += kWave) {
+      const int tt = idx / kWalkCols, jj = idx % kWalkCols;
+      const int cc = cb * kWalkCols + jj;
+      v_s[tt][jj] = (tt < nt && cc < dv) ? to_f32<T>(proj[(size_t)(t0 + tt) * stride + v_off + (size_t)h * dv + cc]) : 0.f;
+    }
+    {
+      const bool live = lane < nt;
+      const float* grow = gates + (size_t)(t0 + (live ? lane : 0)) * gate_stride;
+      if (MODE == WALK_EXP_GATES) {
+        // (F, I) of a stretch of tokens: its summed log forget gates, and what its input gates alone would
+        // make of the maximum; stretches combine as (F1 + F2, max(I1 + F2, I2)).  Lanes beyond the chunk
+        // hold the neutral stretch (0, -inf).
+        float F = 0.f, I = -INFINITY;
+        if (live) {
+          I = cap * tanhf((grow[h] + par0) / cap);
+          F = log_sigmoid_f32(cap * tanhf((grow[nh + h] + par1) / cap));
+        }
+        const float log_i = I, log_f = F;
+#pragma unroll
+        for (int off = 1; off < kWalkChunk; off <<= 1) {
+          const float Fp = __shfl_up(F, off, kWave), Ip = __shfl_up(I, off, kWave);
+          if (lane >= off) {
+            I = fmaxf(Ip + F, I);
+            F = Fp + F;
+          }
+        }
+        const float m_t = fmaxf(m_run + F, I);
+        float m_before = __shfl_up(m_t, 1, kWave);
+        if (lane == 0) m_before = m_run;
+        if (live) {
+          a_s[lane] = expf(log_f + m_before - m_t);
+          b_s[lane] = expf(log_i - m_t);
+          e_s[lane] = expf(-m_t);
+        }
+        m_run = __shfl(m_t, nt - 1, kWave);
+      } else if (live) {
+        const float dt = softplus_f32(grow[h] + par0);
+        a_s[lane] = expf(par1 * dt);
+        b_s[lane] = dt;
+      }
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float a = a_s[tt], b = b_s[tt];
+      const float vj = v_s[tt][j];
+      const float bv = b * vj;
+      float acc = 0.f, nq = 0.f;
+      const float4* k4 = reinterpret_cast<const float4*>(&k_s[tt][0]);
+      const float4* q4 = reinterpret_cast<const float4*>(&q_s[tt][0]);
+#pragma unroll
+      for (int r4 = 0; r4 < RPL / 4; ++r4) {
+        const float4 kk = k4[r4 * 8 + g], qq = q4[r4 * 8 + g];
+        const float kr[4] = {kk.x, kk.y, kk.z, kk.w}, qr[4] = {qq.x, qq.y, qq.z, qq.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int r = r4 * 4 + i;
+          S[r] = fmaf(kr[i], bv, a * S[r]);
+          acc = fmaf(S[r], qr[i], acc);
+          if (MODE == WALK_EXP_GATES) {
+            n[r] = fmaf(kr[i], b, a * n[r]);
+            nq = fmaf(n[r], qr[i], nq);
+          }
+        }
+      }
+      acc += __shfl_xor(acc, 8, kWave);
+      acc += __shfl_xor(acc, 16, kWave);
+      acc += __shfl_xor(acc, 32, kWave);
+      float y;
+      if (MODE == WALK_EXP_GATES) {
+        nq += __shfl_xor(nq, 8, kWave);
+        nq += __shfl_xor(nq, 16, kWave);
+        nq += __shfl_xor(nq, 32, kWave);
+        y = acc / (fmaxf(fabsf(nq), e_s[tt]) + kWalkFloor);
+      } else {
+        y = fmaf(par2, vj, acc);
+      }
+      if (g == 0 && c < dv) out[(size_t)(t0 + tt) * nh * dv + (size_t)h * dv + c] = y;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RPL; ++r) st[r * 64 + lane] = S[r];
+  if (MODE == WALK_EXP_GATES) {
+    if (j == 0) {
+      float4* ndst = reinterpret_cast<float4*>(st + RPL * 64);
+#pragma unroll
+      for (int r4 = 0; r4 < RPL / 4; ++r4) ndst[r4 * 8 + g] = make_float4(n[r4 * 4], n[r4 * 4 + 1], n[r4 * 4 + 2], n[r4 * 4 + 3]);
+    }
+    if (lane == 0) st[RPL * 64 + DKP] = m_run;
+  }
+}
+
+template <typename T, int MODE>
+static int launch_state_walk(const void* proj, int stride, int q_off, int k_off, int v_off, int heads_per_group,
+                             const float* gates, int gate_stride, const float* p0, const float* p1, const float* p2,
+                             float cap, float q_scale, float* state, const int* state_slots, const int* cu_tokens,
+                             float* out, int n_entries, int nh, int dk, int dv, hipStream_t stream) {
+  const int ncb = ceil_div(dv, kWalkCols);
+  dim3 grid(ncb, nh, n_entries);
+#define WALK(RPL)                                                                                                      \
+  state_walk_kernel<T, RPL, MODE><<<grid, kWave, 0, stream>>>((const T*)proj, stride, q_off, k_off, v_off,             \
+                                                              heads_per_group, gates, gate_stride, p0, p1, p2, cap,    \
+                                                              q_scale, state, state_slots, cu_tokens, out, nh, dk, dv, \
+                                                              ncb)
+  if (dk <= 32) WALK(4);
+  else if (dk <= 64) WALK(8);
+  else if (dk <= 128) WALK(16);
+  else if (dk <= 256) WALK(32);
+  else return SHARPI_ERR_ARG;
+#undef WALK
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+// proj [T, stride] (dtype): q and k of head h at columns q_off / k_off + (h / heads_per_group) dk, v at
+// v_off + h dv.  gates float [T, gate_stride]: WALK_EXP_GATES reads columns h (input gate) and nh + h
+// (forget gate), p0 / p1 their biases [nh], cap the gates' cap; WALK_STATE_SPACE reads column h (the
+// step size before its softplus), p0 its bias, p1 A_log, p2 D (all [nh]).  state float [slots, nh,
+// ceil(dv / 8), slice]; out float [T, nh dv].
+SHARPI_EXPORT int sharpi_state_walk(const void* proj, int dtype, int stride, int q_off, int k_off, int v_off,
+                                    int heads_per_group, const float* gates, int gate_stride, const float* p0,
+                                    const float* p1, const float* p2, float cap, float q_scale, int mode, float* state,
+                                    const int* state_slots, const int* cu_tokens, float* out, int n_entries, int nh,
+                                    int dk, int dv, hipStream_t stream) {
+  if (n_entries <= 0) return SHARPI_OK;
+  if (nh <= 0 || nh > 65535 || n_entries > 65535 || dk <= 0 || dk > 256 || dv <= 0 || heads_per_group <= 0) return SHARPI_ERR_ARG;
+  if (mode != WALK_EXP_GATES && mode != WALK_STATE_SPACE) return SHARPI_ERR_ARG;
+  if (!gates || !p0 || !p1 || (mode == WALK_STATE_SPACE && !p2) || (mode == WALK_EXP_GATES && !(cap > 0.f))) return SHARPI_ERR_ARG;
+  if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;
+#define GO(TT, MM)                                                                                                     \
+  return launch_state_walk<TT, MM>(proj, stride, q_off, k_off, v_off, heads_per_group, gates, gate_stride, p0, p1, p2, \
+                                   cap, q_scale, state, state_slots, cu_tokens, out, n_entries, nh, dk, dv, stream)
+  if (mode == WALK_EXP_GATES) {
+    if (dtype == DT_F32) GO(float, WALK_EXP_GATES);
+    GO(bf16_t, WALK_EXP_GATES);
+  }
+  if (dtype == DT_F32) GO(float, WALK_STATE_SPACE);
+  GO(bf16_t, WALK_STATE_SPACE);
+#undef GO
+}
+
+// ---------------------------------------------------------------------------
+// Behind a walk: o float [T, G * gd] in G equal parts, each divided by its root mean square, times a
+// weight per channel, times a gate act(z) read from columns g_off.. of proj [T, stride] (act: 0 none,
+// 1 SiLU, 2 sigmoid).  gate_first: the gate multiplies o BEFORE the statistics are taken (the norm
+// then sees the gated values); otherwise after the weight.  A wave a (token, part).
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float gate_value(int act, float z) {
+  const float s = 1.0f / (1.0f + expf(-z));
+  return act == 1 ? z * s : s;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void group_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w,
+                                                               float eps, const T* __restrict__ proj, int stride,
+                                                               int g_off, int act, int gate_first, T* __restrict__ out,
+                                                               int n_tokens, int G, int gd) {
+  const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);     // (token, part), parts fastest
+  const int lane = threadIdx.x & (kWave - 1);
+  if (pair >= n_tokens * G) return;
+  const int t = pair / G, p = pair % G;
+  const float* x = o + (size_t)pair * gd;
+  const T* gate = act ? proj + (size_t)t * stride + g_off + (size_t)p * gd : nullptr;
+  float ss = 0.f;
+  for (int d = lane; d < gd; d += kWave) {
+    float v = x[d];
+    if (gate && gate_first) v *= gate_value(act, to_f32<T>(gate[d]));
+    ss = fmaf(v, v, ss);
+  }
+  ss = wave_sum(ss);
+  const float inv = rsqrtf(ss / (float)gd + eps);
+  for (int d = lane; d < gd; d += kWave) {
+    float v = x[d];
+    if (gate && gate_first) v *= gate_value(act, to_f32<T>(gate[d]));
+    float y = v * inv * w[(size_t)p * gd + d];
+    if (gate && !gate_first) y *= gate_value(act, to_f32<T>(gate[d]));
+    out[(size_t)pair * gd + d] = from_f32<T>(y);
+  }
+}
+
+SHARPI_EXPORT int sharpi_group_norm_gate(const float* o, const float* w, float eps, const void* proj, int dtype,
+                                         int stride, int g_off, int act, int gate_first, void* out, int n_tokens, int G,
+                                         int gd, hipStream_t stream) {
+  if (n_tokens <= 0) return SHARPI_OK;
+  if (G <= 0 || gd <= 0 || act < 0 || act > 2 || (act && !proj)) return SHARPI_ERR_ARG;
+  const int blocks = ceil_div(n_tokens * G, 4);
+  if (dtype == DT_F32)
+    group_norm_gate_kernel<float><<<blocks, 256, 0, stream>>>(o, w, eps, (const float*)proj, stride, g_off, act, gate_first,
+                                                               (float*)out, n_tokens, G, gd);
+  else if (dtype == DT_BF16)
+    group_norm_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>(o, w, eps, (const bf16_t*)proj, stride, g_off, act,
+                                                                gate_first, (bf16_t*)out, n_tokens, G, gd);
+  else
+    return SHARPI_ERR_ARG;
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// A short causal convolution over time on C channels of proj [T, stride] (columns c_off..), with a
+// bias, then SiLU: y_t = silu(b + sum_j w[:, j] u_(t - taps + 1 + j)) (w float [C, taps]; the last
+// column is the current token's).  Before an entry's first row of the step the inputs come from the
+// request's tail, float [slots, taps - 1, C] (its last taps - 1 inputs, oldest first; zeros for a new
+// request).  A second kernel moves the tails on.  Sums in float, the current token's term last.
+// ---------------------------------------------------------------------------
+constexpr int kConvMaxTaps = 8;
+
+template <typename T>
+__global__ __launch_bounds__(256) void short_conv_kernel(const T* __restrict__ proj, int stride, int c_off,
+                                                          const float* __restrict__ w, const float* __restrict__ bias,
+                                                          int taps, const float* __restrict__ tail,
+                                                          const int* __restrict__ state_slots,
+                                                          const int* __restrict__ entry_of_token,
+                                                          const int* __restrict__ cu_tokens, T* __restrict__ out, int C) {
+  const int t = blockIdx.x;
+  const int ch = blockIdx.y * blockDim.x + threadIdx.x;
+  if (ch >= C) return;
+  const int e = entry_of_token[t];
+  const int local = t - cu_tokens[e];
+  const float* tl = tail ? tail + (size_t)state_slots[e] * (taps - 1) * C : nullptr;
+  float acc = bias ? bias[ch] : 0.f;
+  for (int jx = 0; jx < taps; ++jx) {
+    const int back = taps - 1 - jx;           // how many tokens before this one
+    float u;
+    if (back <= local) u = to_f32<T>(proj[(size_t)(t - back) * stride + c_off + ch]);
+    else u = tl[(size_t)(taps - 1 + local - back) * C + ch];
+    acc = fmaf(w[(size_t)ch * taps + jx], u, acc);
+  }
+  out[(size_t)t * C + ch] = from_f32<T>(acc / (1.0f + expf(-acc)));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void short_conv_tail_kernel(const T* __restrict__ proj, int stride, int c_off, int taps,
+                                                               float* __restrict__ tail, const int* __restrict__ state_slots,
+                                                               const int* __restrict__ cu_tokens, int C) {
+  const int e = blockIdx.x;
+  const int ch = blockIdx.y * blockDim.x + threadIdx.x;
+  if (ch >= C) return;
+  const int first = cu_tokens[e], L = cu_tokens[e + 1] - first;
+  if (L <= 0) return;
+  float* tl = tail + (size_t)state_slots[e] * (taps - 1) * C;
+  float keep[kConvMaxTaps];
+  for (int i = 0; i < taps - 1; ++i) {        // the new row i is the input at local index L - (taps - 1) + i
+    const int li = L - (taps - 1) + i;
+    keep[i] = li >= 0 ? to_f32<T>(proj[(size_t)(first + li) * stride + c_off + ch]) : tl[(size_t)(taps - 1 + li) * C + ch];
+  }
+  for (int i = 0; i < taps - 1; ++i) tl[(size_t)i * C + ch] = keep[i];
+}
+
+SHARPI_EXPORT int sharpi_short_conv(const void* proj, int dtype, int stride, int c_off, const float* w, const float* bias,
+                                    int taps, float* tail, const int* state_slots, const int* entry_of_token,
+                                    const int* cu_tokens, void* out, int n_tokens, int n_entries, int C, int update_tail,
+                                    hipStream_t stream) {
+  if (n_tokens <= 0) return SHARPI_OK;
+  if (C <= 0 || taps < 1 || taps > kConvMaxTaps || (taps > 1 && !tail) || n_entries <= 0 || ceil_div(C, 256) > 65535) return SHARPI_ERR_ARG;
+  if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;
+  dim3 grid(n_tokens, ceil_div(C, 256)), tgrid(n_entries, ceil_div(C, 256));
+  if (dtype == DT_F32) {
+    short_conv_kernel<float><<<grid, 256, 0, stream>>>((const float*)proj, stride, c_off, w, bias, taps, tail, state_slots,
+                                                        entry_of_token, cu_tokens, (float*)out, C);
+    SHARPI_CHECK_LAUNCH();
+    if (taps > 1 && update_tail)
+      short_conv_tail_kernel<float><<<tgrid, 256, 0, stream>>>((const float*)proj, stride, c_off, taps, tail, state_slots,
+                                                                cu_tokens, C);
+  } else {
+    short_conv_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)proj, stride, c_off, w, bias, taps, tail,
+                                                         state_slots, entry_of_token, cu_tokens, (bf16_t*)out, C);
+    SHARPI_CHECK_LAUNCH();
+    if (taps > 1 && update_tail)
+      short_conv_tail_kernel<bf16_t><<<tgrid, 256, 0, stream>>>((const bf16_t*)proj, stride, c_off, taps, tail, state_slots,
+                                                                 cu_tokens, C);
+  }
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}

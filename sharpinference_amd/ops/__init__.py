@@ -153,16 +153,19 @@ def add_rmsnorm(h: torch.Tensor, delta, weight: Optional[torch.Tensor], eps: flo
     return out
 
 
-def gated_act(gate_up: torch.Tensor, scale: Optional[torch.Tensor] = None, act: int = ACT_SILU) -> torch.Tensor:
+def gated_act(gate_up: torch.Tensor, scale: Optional[torch.Tensor] = None, act: int = ACT_SILU,
+              bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """[M, 2I] (gate columns, then up columns) -> act(s*g) * (s*u) [M, I]; act: ACT_SILU or
-    ACT_GELU_TANH."""
-    _dev(gate_up, scale)
+    ACT_GELU_TANH.  ``bias`` (float32 [2I]) is added to the gate and up columns first, in float."""
+    _dev(gate_up, scale, bias)
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (gate_up.shape[1],), "gated_act: bias must be float32 [2I]")
     _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "gated_act: input must be [M, 2I]")
     M, I2 = gate_up.shape
     if scale is not None:
         _need(scale.dtype == torch.float32 and scale.shape == (M,), "gated_act: scale must be float32 [M]")
     out = torch.empty(M, I2 // 2, dtype=gate_up.dtype, device=gate_up.device)
-    _run("sharpi_silu_mul", _ptr(gate_up), _ptr(scale), _ptr(out), _code(gate_up.dtype), M, I2 // 2, int(act), _stream())
+    _run("sharpi_silu_mul", _ptr(gate_up), _ptr(scale), _ptr(out), _code(gate_up.dtype), M, I2 // 2, int(act), _ptr(bias), _stream())
     return out
 
 
@@ -235,22 +238,25 @@ PAIRS_INTERLEAVED, PAIRS_HALF_SPLIT = 0, 1
 def rope_kv(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
             positions: torch.Tensor, inv_freq: Optional[torch.Tensor], qk_norm: bool, eps: float,
             temperature: Optional[Tuple[float, float]], nh: int, nkv: int, hd: int,
-            pair_layout: int = PAIRS_INTERLEAVED, bias: Optional[torch.Tensor] = None, vd: Optional[int] = None) -> torch.Tensor:
+            pair_layout: int = PAIRS_INTERLEAVED, bias: Optional[torch.Tensor] = None, vd: Optional[int] = None,
+            extra_columns: int = 0) -> torch.Tensor:
     """Rotate / norm / scale the heads of qkv [T, (nh+nkv)*hd + nkv*vd] (vd, the values' width, is hd
     unless given); K and V go into the layer's
     cache [pages, nkv, page_size, hd] at slot_mapping; returns q [T, nh*hd].  inv_freq [r/2]
     rotates the first r <= hd elements of every head, in pairs (2i, 2i+1) or (i, i + r/2)
     (``pair_layout``); the rest of the head passes through.  ``bias`` (float32, one value per
-    column of qkv) is added to every row first, in float."""
+    column of q, k and v) is added to every row first, in float.  ``extra_columns``: further columns of
+    each row behind q, k and v (another product's outputs made by the same launch), which are left alone."""
     _dev(qkv, k_cache, v_cache, slot_mapping, positions, inv_freq, bias)
     if bias is not None:
-        _need(bias.dtype == torch.float32 and bias.shape == (qkv.shape[1],) and bias.is_contiguous(),
+        _need(bias.dtype == torch.float32 and bias.shape == (qkv.shape[1] - extra_columns,) and bias.is_contiguous(),
               "rope_kv: bias must be float32, one value per column of qkv")
     _i32(slot_mapping, "slot_mapping")
     _i32(positions, "positions")
     T = qkv.shape[0]
     vd = int(vd or hd)
-    _need(qkv.dim() == 2 and qkv.shape[1] == (nh + nkv) * hd + nkv * vd, "rope_kv: qkv must be [T, (nh+nkv)*hd + nkv*vd]")
+    _need(qkv.dim() == 2 and extra_columns >= 0 and qkv.shape[1] == (nh + nkv) * hd + nkv * vd + extra_columns,
+          "rope_kv: qkv must be [T, (nh+nkv)*hd + nkv*vd (+ extra_columns)]")
     _need(_cache_shapes_ok(k_cache, v_cache, nkv, hd, vd), "rope_kv: caches must be K [pages, nkv, page_size, hd], V [pages, nkv, vd, page_size]")
     _need(k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype, "rope_kv: cache dtype differs from qkv's")
     _need(slot_mapping.shape == (T,) and positions.shape == (T,), "rope_kv: slot_mapping / positions must be [T]")
@@ -266,8 +272,21 @@ def rope_kv(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slo
     _run("sharpi_rope_kv", _ptr(qkv), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _code(qkv.dtype),
          _ptr(slot_mapping), _ptr(positions), _ptr(inv_freq), _ptr(bias), 1 if qk_norm else 0, float(eps),
          1 if temperature is not None else 0, float(fs), float(asc), T, nh, nkv, hd, vd, page_size, int(pair_layout),
-         rotary_dim, _stream())
+         rotary_dim, qkv.shape[1], _stream())
     return q_out
+
+
+def _sink_args(sink, nh: int):
+    """The two arguments the attention kernels take for a sink: (flag, values).  ``sink`` False / None: no
+    sink; True: one more term exp(0) in the denominator; a float32 tensor [nh]: exp(sink[head]), a
+    learned score per head (not scaled, without a value)."""
+    if sink is None or sink is False:
+        return 0, None
+    if sink is True:
+        return 1, None
+    _dev(sink)
+    _need(sink.dtype == torch.float32 and sink.shape == (nh,), "attention: a learned sink must be float32 [nh]")
+    return 1, _ptr(sink)
 
 
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
@@ -292,7 +311,7 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     out = torch.empty(T, nh * vd, dtype=q.dtype, device=q.device)
     _run("sharpi_attention_generic", _ptr(q), _ptr(k_cache), _ptr(v_cache), _code(q.dtype), _ptr(block_table),
          _ptr(entry_of_token), _ptr(positions), _ptr(out), int(window_kind), int(window), float(scale), T, nh, nkv,
-         hd, vd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], float(softcap), 1 if sink else 0, _stream())
+         hd, vd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], float(softcap), *_sink_args(sink, nh), _stream())
     return out
 
 
@@ -337,7 +356,7 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     _run("sharpi_attention_decode", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(entry_of_token),
          _ptr(positions), _ptr(token_list), _ptr(part_o), _ptr(part_ml), _ptr(out), int(window_kind), int(window),
          float(scale), n_list, nh, nkv, hd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], max_splits,
-         float(softcap), 1 if sink else 0, _stream())
+         float(softcap), *_sink_args(sink, nh), _stream())
     return out
 
 
@@ -372,7 +391,7 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _need(out.shape == q.shape and out.dtype == q.dtype, "attention_prefill: out must match q")
     _run("sharpi_attention_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(positions),
          _ptr(tiles), _ptr(out), tiles.shape[0], int(tile_tokens), int(window_kind), int(window), float(scale), nh,
-         nkv, hd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], float(softcap), 1 if sink else 0, _stream())
+         nkv, hd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], float(softcap), *_sink_args(sink, nh), _stream())
     return out
 
 
@@ -1404,11 +1423,11 @@ def norm_mean(xs, weights, eps: float) -> torch.Tensor:
 # ---------------------------------------------------------------------------
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, group, ctx, window_kind: int,
               window: int, scale: float, nh: int, nkv: int, hd: int, vd: Optional[int] = None, softcap: float = 0.0,
-              sink: bool = False) -> torch.Tensor:
+              sink=False) -> torch.Tensor:
     """Attention of the step's tokens over their requests' pages (`group`: the cache group's
     block tables, `ctx`: the step).  Values of another width than keys (vd) go through the float kernel.
     softcap > 0 caps the scores (softcap * tanh(score / softcap)); sink adds a key of score 0 without a
-    value to the softmax's denominator."""
+    value to the softmax's denominator (True), or one of a learned score per head (a float32 tensor [nh])."""
     same = vd is None or vd == hd
     if same and decode_attention_ok(q.dtype, hd) and (prefill_attention_ok(q.dtype, hd) or not ctx.n_prefill_tiles):
         # entries of one token: split-K decode kernel; longer entries: flash kernel, a tile of tokens a block
@@ -1489,3 +1508,192 @@ def measured_peaks(device="cuda:0", read_bytes: int = 4 << 30, repeats: int = 5)
         best_mfma = min(best_mfma, a.elapsed_time(b))
     flops = blocks * 4 * iters * 8 * (2.0 * 16 * 16 * 32)
     return {"hbm_gbs": done.value / best_read / 1e6, "bf16_tflops": flops / best_mfma / 1e9}
+
+
+# ---------------------------------------------------------------------------
+# recurrent states with a scalar decay per (token, head); gated branches; a second input from the token
+# ---------------------------------------------------------------------------
+WALK_EXP_GATES, WALK_STATE_SPACE = 0, 1      # csrc/state_walk.hip
+WALK_MAX_KEY_DIM = 256
+WALK_STATE_COLS = _lib.WALK_STATE_COLS
+SHORT_CONV_MAX_TAPS = 8                       # csrc/state_walk.hip kConvMaxTaps
+GATE_NONE, GATE_SILU, GATE_SIGMOID_ACT = 0, 1, 2
+
+
+def _walk_rows(dk: int) -> int:
+    return 32 if dk <= 32 else 64 if dk <= 64 else 128 if dk <= 128 else 256
+
+
+def walk_state_shape(nh: int, dk: int, dv: int, mode: int) -> tuple:
+    """A request's recurrent state as the walk keeps it: [heads, ceil(dv / 8), slice].  A slice holds 8
+    value columns: DKP x 8 floats of the matrix (DKP = dk rounded up to 32 / 64 / 128 / 256; row
+    g * (DKP / 8) + r of column j at r * 64 + 8 g + j) and, with exponential gates, DKP floats of the
+    normaliser vector (four rows of a row group together, the groups side by side) and 8 floats that
+    begin with the running maximum."""
+    dkp = _walk_rows(dk)
+    return (nh, (dv + WALK_STATE_COLS - 1) // WALK_STATE_COLS, dkp * 8 + (dkp + 8 if mode == WALK_EXP_GATES else 0))
+
+
+def walk_state_matrices(state: torch.Tensor, dk: int, dv: int, mode: int):
+    """The state as kept -> (S [.., heads, dk, dv], n [.., heads, dk] or None, m [.., heads] or None): copies, for
+    tests and tools (the normaliser and the maximum are read from every head's first slice)."""
+    *lead, nh, ncb, _ = state.shape
+    dkp = _walk_rows(dk)
+    rpl = dkp // 8
+    S = state[..., : dkp * 8].reshape(*lead, nh, ncb, rpl, 8, 8)          # [.., h, slice, r, g, j]
+    S = S.movedim(-2, -3).reshape(*lead, nh, ncb, dkp, 8)               # row g * rpl + r
+    S = S.movedim(-3, -2).reshape(*lead, nh, dkp, ncb * 8)[..., :dk, :dv].contiguous()
+    if mode != WALK_EXP_GATES:
+        return S, None, None
+    n = state[..., 0, dkp * 8: dkp * 8 + dkp].reshape(*lead, nh, rpl // 4, 8, 4)     # [.., h, r4, g, i]
+    n = n.movedim(-2, -3).reshape(*lead, nh, dkp)[..., :dk].contiguous()
+    return S, n, state[..., 0, dkp * 8 + dkp].contiguous()
+
+
+def state_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, heads_per_group: int, gates: torch.Tensor,
+               params, cap: float, q_scale: float, mode: int, state: torch.Tensor, ctx, nh: int, dk: int, dv: int) -> torch.Tensor:
+    """The recurrence S_t = a_t S_(t-1) + b_t k_t v_t^T, o_t = S_t^T q_t per head with one decay a_t and one
+    input weight b_t per (token, head), token by token along every entry of the step, from and into
+    state [slots, *walk_state_shape(nh, dk, dv, mode)] (float32) at the entries' state slots.  q and k of
+    head h are columns q_off / k_off + (h // heads_per_group) * dk of proj [T, N], v columns v_off + h * dv;
+    q is multiplied by q_scale.  ``gates`` float32 [T, M] and ``params`` (float32 [nh] each):
+
+    * WALK_EXP_GATES: gates columns h and nh + h are the input and forget gates' pre-activations, params
+      (input bias, forget bias); i = cap tanh((x + b) / cap), f = log_sigmoid(cap tanh(...)), a running
+      maximum m (starting at 0) keeps the exponentials in range, a normaliser vector n moves beside S,
+      and the result is o / (max(|n . q|, exp(-m)) + 1e-6);
+    * WALK_STATE_SPACE: gates column h is the step size before its softplus, params (its bias, A_log, D);
+      a = exp(-exp(A_log) dt), b = dt, and the result is o + D v.
+
+    Returns float32 [T, nh * dv]."""
+    _dev(proj, gates, state, *params)
+    T, N = proj.shape
+    groups = nh // heads_per_group if heads_per_group > 0 else 0
+    _need(1 <= dk <= WALK_MAX_KEY_DIM and dv >= 1 and nh >= 1 and heads_per_group >= 1 and nh % heads_per_group == 0,
+          f"state_walk: key channels 1..{WALK_MAX_KEY_DIM}, heads a multiple of the heads a group")
+    _need(min(q_off, k_off, v_off) >= 0 and max(q_off, k_off) + groups * dk <= N and v_off + nh * dv <= N,
+          "state_walk: q, k and v columns must lie inside proj")
+    _need(mode in (WALK_EXP_GATES, WALK_STATE_SPACE), "state_walk: mode 0 (exponential gates) or 1 (state space)")
+    n_par, n_cols = (2, 2 * nh) if mode == WALK_EXP_GATES else (3, nh)
+    _need(gates.dtype == torch.float32 and gates.dim() == 2 and gates.shape[0] == T and gates.shape[1] >= n_cols,
+          f"state_walk: gates float32 [T, >= {n_cols}] wanted")
+    _need(len(params) == n_par and all(p.dtype == torch.float32 and p.shape == (nh,) for p in params),
+          f"state_walk: {n_par} float32 [nh] parameter vectors wanted")
+    _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == walk_state_shape(nh, dk, dv, mode),
+          "state_walk: state must be float32 [slots, *walk_state_shape(nh, dk, dv, mode)]")
+    _need(ctx.state_slots.shape == (ctx.n_entries,) and ctx.cu_tokens.shape == (ctx.n_entries + 1,) and ctx.n_tokens == T,
+          "state_walk: the step's per-entry arrays do not fit")
+    out = torch.empty(T, nh * dv, dtype=torch.float32, device=proj.device)
+    p = list(params) + [None] * (3 - n_par)
+    _run("sharpi_state_walk", _ptr(proj), _code(proj.dtype), N, int(q_off), int(k_off), int(v_off), int(heads_per_group),
+         _ptr(gates), gates.shape[1], _ptr(p[0]), _ptr(p[1]), _ptr(p[2]), float(cap), float(q_scale), int(mode), _ptr(state),
+         _ptr(ctx.state_slots), _ptr(ctx.cu_tokens), _ptr(out), ctx.n_entries, nh, dk, dv, _stream())
+    return out
+
+
+def group_norm_gate(o: torch.Tensor, weight: torch.Tensor, eps: float, groups: int, out_dtype: torch.dtype,
+                    gate_proj: Optional[torch.Tensor] = None, gate_off: int = 0, gate_act: int = GATE_NONE,
+                    gate_first: bool = False) -> torch.Tensor:
+    """o float32 [T, N] in `groups` equal parts, each divided by its root mean square, times weight
+    (float32 [N]), times act(gate) (columns gate_off.. of gate_proj [T, M], of out_dtype; act GATE_SILU
+    or GATE_SIGMOID_ACT).  ``gate_first``: the gate multiplies o before the statistics are taken."""
+    _dev(o, weight, gate_proj)
+    T, N = o.shape
+    _need(o.dtype == torch.float32 and groups >= 1 and N % groups == 0 and weight.dtype == torch.float32 and weight.shape == (N,),
+          "group_norm_gate: o float32 [T, N], N a multiple of the groups, weight float32 [N]")
+    _need(gate_act in (GATE_NONE, GATE_SILU, GATE_SIGMOID_ACT), "group_norm_gate: gate_act 0, 1 or 2")
+    stride = 0
+    if gate_act != GATE_NONE:
+        _need(gate_proj is not None and gate_proj.dtype == out_dtype and gate_proj.dim() == 2 and gate_proj.shape[0] == T
+              and 0 <= gate_off and gate_off + N <= gate_proj.shape[1], "group_norm_gate: the gate's columns must lie inside gate_proj")
+        stride = gate_proj.shape[1]
+    out = torch.empty(T, N, dtype=out_dtype, device=o.device)
+    _run("sharpi_group_norm_gate", _ptr(o), _ptr(weight), float(eps), _ptr(gate_proj) if gate_act else None, _code(out_dtype),
+         stride, int(gate_off), int(gate_act), 1 if gate_first else 0, _ptr(out), T, groups, N // groups, _stream())
+    return out
+
+
+def short_conv(proj: torch.Tensor, c_off: int, channels: int, weight: torch.Tensor, bias: Optional[torch.Tensor],
+               tail: Optional[torch.Tensor], ctx, update_tail: bool = True) -> torch.Tensor:
+    """silu(bias + causal convolution over time) on `channels` columns of proj [T, N] from c_off: weight
+    float32 [channels, taps] (the last column is the current token's), bias float32 [channels] or None; tail
+    float32 [slots, taps - 1, channels] carries each request's last inputs from step to step (None when
+    taps is 1) and is brought up to date unless update_tail is False.  Returns [T, channels] of proj's dtype."""
+    _dev(proj, weight, bias, tail)
+    T, N = proj.shape
+    taps = weight.shape[1] if weight.dim() == 2 else 0
+    _need(weight.dtype == torch.float32 and weight.shape == (channels, taps) and 1 <= taps <= SHORT_CONV_MAX_TAPS,
+          f"short_conv: weight must be float32 [channels, 1..{SHORT_CONV_MAX_TAPS} taps]")
+    _need(0 <= c_off and c_off + channels <= N, "short_conv: the channels must lie inside proj")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (channels,)), "short_conv: bias must be float32 [channels]")
+    if taps > 1:
+        _need(tail is not None and tail.dtype == torch.float32 and tail.dim() == 3 and tuple(tail.shape[1:]) == (taps - 1, channels),
+              "short_conv: tail must be float32 [slots, taps - 1, channels]")
+    _need(ctx.state_slots.shape == (ctx.n_entries,) and ctx.cu_tokens.shape == (ctx.n_entries + 1,)
+          and ctx.entry_of_token.shape == (T,), "short_conv: the step's per-entry arrays do not fit")
+    out = torch.empty(T, channels, dtype=proj.dtype, device=proj.device)
+    _run("sharpi_short_conv", _ptr(proj), _code(proj.dtype), N, int(c_off), _ptr(weight), _ptr(bias), taps,
+         _ptr(tail) if taps > 1 else None, _ptr(ctx.state_slots), _ptr(ctx.entry_of_token), _ptr(ctx.cu_tokens), _ptr(out),
+         T, ctx.n_entries, channels, 1 if update_tail else 0, _stream())
+    return out
+
+
+def sigmoid_gate(x: torch.Tensor, gate_proj: torch.Tensor, gate_off: int) -> torch.Tensor:
+    """x [T, N] * sigmoid(gate), the gate columns gate_off.. of gate_proj [T, M] (same dtype)."""
+    _dev(x, gate_proj)
+    T, N = x.shape
+    _need(gate_proj.dtype == x.dtype and gate_proj.dim() == 2 and gate_proj.shape[0] == T and 0 <= gate_off
+          and gate_off + N <= gate_proj.shape[1], "sigmoid_gate: the gate's columns must lie inside gate_proj")
+    out = torch.empty_like(x)
+    _run("sharpi_sigmoid_gate", _ptr(x), _ptr(gate_proj), _code(x.dtype), gate_proj.shape[1], int(gate_off), _ptr(out), T, N, _stream())
+    return out
+
+
+class BranchSum:
+    """Stands for a sum of branch outputs with a scale each, sum_b scales[b] * xs[b], still to be formed
+    (in float): [T, N].  ``stream_add`` folds it into the residual sum; ``tensor()`` forms it alone."""
+
+    def __init__(self, xs, scales):
+        self.xs, self.scales = list(xs), [float(s) for s in scales]
+        self.shape, self.dtype = tuple(xs[0].shape), torch.float32
+
+    def tensor(self) -> torch.Tensor:
+        h = torch.zeros(self.shape, dtype=torch.float32, device=self.xs[0].device)
+        stream_add(h, self)
+        return h
+
+
+def stream_add(h: torch.Tensor, delta, out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """h (float32 [T, N]) += delta in place, in float; delta a tensor [T, N], a BranchSum (up to 4 scaled
+    branches, added in their order) or None.  With ``out_dtype`` the new h is also returned in that
+    storage type."""
+    import ctypes
+
+    xs = delta.xs if isinstance(delta, BranchSum) else [] if delta is None else [delta]
+    scales = delta.scales if isinstance(delta, BranchSum) else [1.0] * len(xs)
+    _dev(h, *xs)
+    _need(h.dim() == 2 and h.dtype == torch.float32 and len(xs) <= 4, "stream_add: h float32 [T, N], at most 4 branches")
+    for x in xs:
+        _need(tuple(x.shape) == tuple(h.shape) and x.dtype == xs[0].dtype, "stream_add: branches of h's shape and of one dtype")
+    n = len(xs)
+    out = torch.empty(h.shape, dtype=out_dtype, device=h.device) if out_dtype is not None else None
+    xp = (ctypes.c_void_p * max(n, 1))(*[x.data_ptr() for x in xs])
+    sp = (ctypes.c_float * max(n, 1))(*scales)
+    _run("sharpi_stream_add", _ptr(h), ctypes.cast(xp, ctypes.c_void_p), ctypes.cast(sp, ctypes.c_void_p), n,
+         _code(xs[0].dtype) if xs else (_code(out_dtype) if out_dtype is not None else 0), _ptr(out),
+         _code(out_dtype) if out_dtype is not None else 0, h.numel(), _stream())
+    return out
+
+
+def side_gate(gate: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, col_off: int) -> torch.Tensor:
+    """gelu_tanh(gate [T, D]) * table[ids[t], col_off : col_off + D]: a slice of each token's row of a side
+    table, gated element by element."""
+    _dev(gate, ids, table)
+    _i32(ids, "ids")
+    T, D = gate.shape
+    _need(ids.shape == (T,) and table.dim() == 2 and 0 <= col_off and col_off + D <= table.shape[1],
+          "side_gate: ids [T]; the slice must lie inside the table's rows")
+    out = torch.empty_like(gate)
+    _run("sharpi_side_gate", _ptr(gate), _code(gate.dtype), _ptr(ids), _ptr(table), _code(table.dtype), table.shape[1],
+         int(col_off), _ptr(out), T, D, _stream())
+    return out

@@ -20,17 +20,17 @@ _SIGNATURES = {
     "sharpi_embed_gather": [P, P, I, P, I, I, F, P],
     "sharpi_scale_softcap": [P, c_longlong, F, F, P],
     "sharpi_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, P, P, P, I, P],
-    "sharpi_silu_mul": [P, P, P, I, I, I, I, P],
+    "sharpi_silu_mul": [P, P, P, I, I, I, I, P, P],
     "sharpi_moe_combine": [P, P, P, P, P, I, I, I, I, P],
     "sharpi_cast": [P, I, P, I, c_longlong, P],
     "sharpi_add_bias": [P, I, P, I, I, P],
     "sharpi_peak_read": [P, c_longlong, P, P, P],
     "sharpi_peak_mfma": [P, I, I, P],
     "sharpi_random_fill": [P, I, c_longlong, c_ulonglong, I, F, I, I, P],
-    "sharpi_rope_kv": [P, P, P, P, I, P, P, P, P, I, F, I, F, F, I, I, I, I, I, I, I, I, P],
-    "sharpi_attention_generic": [P, P, P, I, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, F, I, P],
-    "sharpi_attention_decode": [P, P, P, P, P, P, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, F, I, P],
-    "sharpi_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, F, I, I, I, I, I, I, F, I, P],
+    "sharpi_rope_kv": [P, P, P, P, I, P, P, P, P, I, F, I, F, F, I, I, I, I, I, I, I, I, I, P],
+    "sharpi_attention_generic": [P, P, P, I, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, F, I, P, P],
+    "sharpi_attention_decode": [P, P, P, P, P, P, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, F, I, P, P],
+    "sharpi_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, F, I, I, I, I, I, I, F, I, P, P],
     "sharpi_gemm_tiled": [P, P, P, I, I, I, I, I, P, P, I, P],
     "sharpi_gemm_skinny": [P, P, P, I, I, I, I, P, P, I, I, I, I, I, P],
     "sharpi_gemm_skinny_swiglu": [P, P, P, I, I, I, P, P, I, P, I, I, I, I, I, P],
@@ -58,6 +58,12 @@ _SIGNATURES = {
     "sharpi_activation": [P, P, I, c_longlong, I, P],
     "sharpi_norm_mean": [P, P, I, I, P, I, I, F, P],
     "sharpi_post_pre_norm": [P, P, P, I, I, P, P, P, I, I, I, F, P],
+    "sharpi_state_walk": [P, I, I, I, I, I, I, P, I, P, P, P, F, F, I, P, P, P, P, I, I, I, I, P],
+    "sharpi_group_norm_gate": [P, P, F, P, I, I, I, I, I, P, I, I, I, P],
+    "sharpi_short_conv": [P, I, I, I, P, P, I, P, P, P, P, P, I, I, I, I, P],
+    "sharpi_sigmoid_gate": [P, P, I, I, I, P, I, I, P],
+    "sharpi_stream_add": [P, P, P, I, I, P, I, c_longlong, P],
+    "sharpi_side_gate": [P, I, P, P, I, I, I, P, I, I, P],
 }
 
 # entry points that newer sources add; bound when present
@@ -71,6 +77,7 @@ PICKED_MAX_PAIRS = 64       # (token, pick) pairs the few-rows product takes str
 FUSED_NORM_ROUTER_MAX_HIDDEN = 8192   # widest row of the norm + router kernel
 ROUTER_MAX_EXPERTS = 1024   # experts the routing kernels hold scores for
 GLA_STATE_COLS = 8          # value columns of a linear-attention state that lie together in memory
+WALK_STATE_COLS = 8         # value columns of a slice of a scalar-decay recurrent state (csrc/state_walk.hip)
 _BUILT_WITH = {
     "sharpi_attention_decode_split_keys": DECODE_RUN_KEYS,
     "sharpi_attention_prefill_tile_tokens": PREFILL_TILE_TOKENS,
@@ -78,6 +85,7 @@ _BUILT_WITH = {
     "sharpi_gemm_skinny_max_picked": PICKED_MAX_PAIRS,
     "sharpi_add_rmsnorm_router_max_hidden": FUSED_NORM_ROUTER_MAX_HIDDEN,
     "sharpi_gla_state_cols": GLA_STATE_COLS,
+    "sharpi_state_walk_cols": WALK_STATE_COLS,
 }
 
 

@@ -75,20 +75,25 @@ class Attention(Part):
     (weights [channels, n]; zeros before a sequence's start; the last n - 1 projected rows of a
     request are carried in its state slot).  ``softcap`` c: scores become c tanh(score / c).
     ``sink``: the softmax's denominator holds one more term exp(0), a key of score 0 that has no
-    value.  A rotary object's ``magnitude`` multiplies cos and sin.  ``names``: the tensors' names
-    behind the layer's prefix."""
+    value; ``sink="learned"``: the term is exp(s_h) with a stored number s_h per head (tensor
+    ``sink`` [heads], float; not scaled).  ``gate``: the heads' outputs side by side are multiplied
+    element by element by sigmoid(W_g x) (W_g [heads * v_head_dim, hidden], a product of the same
+    input as q, k and v, made by the same launch) before the output projection.  A rotary object's
+    ``magnitude`` multiplies cos and sin.  ``names``: the tensors' names behind the layer's prefix."""
 
     NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
              "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
              "q_norm": "q_norm.weight", "k_norm": "k_norm.weight",
-             "q_conv": "q_conv.weight", "k_conv": "k_conv.weight", "v_conv": "v_conv.weight"}
+             "q_conv": "q_conv.weight", "k_conv": "k_conv.weight", "v_conv": "v_conv.weight",
+             "sink": "sink", "g": "g_proj.weight"}
 
     def __init__(self, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  rotary=None, qk_norm_eps: Optional[float] = None,
                  q_temperature: Optional[Tuple[float, float]] = None, window_kind: int = WINDOW_NONE,
                  window: int = 0, scale: Optional[float] = None, bias: bool = False, o_bias: Optional[bool] = None,
                  v_head_dim: Optional[int] = None, qk_norm_weights: Optional[str] = None, values_from_keys: bool = False,
-                 conv_taps: int = 0, softcap: float = 0.0, sink: bool = False, names: Optional[Dict[str, str]] = None):
+                 conv_taps: int = 0, softcap: float = 0.0, sink=False, names: Optional[Dict[str, str]] = None,
+                 gate: bool = False):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads cannot share {num_kv_heads} kv heads")
         prep = bool(qk_norm_weights or values_from_keys or conv_taps)
@@ -120,7 +125,12 @@ class Attention(Part):
         if self.conv_taps and not 2 <= self.conv_taps <= ops.QK_PREP_MAX_TAPS:
             raise ValueError(f"a convolution of {conv_taps} taps is not taken: 2 to {ops.QK_PREP_MAX_TAPS}")
         self.qk_norm_weights, self.values_from_keys = qk_norm_weights, bool(values_from_keys)
+        if sink not in (False, True, None, "learned"):
+            raise ValueError(f"sink {sink!r} is not known (False, True, 'learned')")
         self.softcap, self.sink = float(softcap or 0.0), bool(sink)
+        self.learned_sink, self.has_gate = sink == "learned", bool(gate)
+        if self.has_gate and prep:
+            raise ValueError("an output gate belongs to the rotate-then-norm form of the layer")
         if self.softcap < 0:
             raise ValueError("softcap must be positive (or 0 for none)")
         self.prep = prep                                         # the layer takes the norm-before-rotation kernel
@@ -139,6 +149,7 @@ class Attention(Part):
         self.w_q_norm: Optional[torch.Tensor] = None             # float32
         self.w_k_norm: Optional[torch.Tensor] = None
         self.w_conv: Optional[torch.Tensor] = None               # float32 [q + k + v channels, taps]
+        self.w_sink: Optional[torch.Tensor] = None               # float32 [heads]
 
     # -- what it needs --------------------------------------------------------
     def step_planners(self):
@@ -174,6 +185,10 @@ class Attention(Part):
             whole = self.qk_norm_weights == "projection"
             specs[prefix + n["q_norm"]] = ParamSpec((q if whole else self.hd,), INIT_NORM_WEIGHT)
             specs[prefix + n["k_norm"]] = ParamSpec((kv if whole else self.hd,), INIT_NORM_WEIGHT)
+        if self.learned_sink:
+            specs[prefix + n["sink"]] = ParamSpec((self.nh,))
+        if self.has_gate:
+            specs[prefix + n["g"]] = ParamSpec((ov, self.hidden))
         if self.conv_taps:
             specs[prefix + n["q_conv"]] = ParamSpec((q, self.conv_taps))
             specs[prefix + n["k_conv"]] = ParamSpec((kv, self.conv_taps))
@@ -184,7 +199,7 @@ class Attention(Part):
     def load(self, prefix: str, source: TensorSource) -> None:
         n = self.names
         kinds = ("q", "k") if self.values_from_keys else ("q", "k", "v")
-        parts = [source.get(prefix + n[k]) for k in kinds]
+        parts = [source.get(prefix + n[k]) for k in kinds + (("g",) if self.has_gate else ())]
         dt = torch.float32 if any(p.dtype == torch.float32 for p in parts) else parts[0].dtype
         fused = torch.empty(sum(p.shape[0] for p in parts), self.hidden, dtype=dt, device=parts[0].device)
         o = 0
@@ -201,6 +216,8 @@ class Attention(Part):
         if self.qk_norm_weights:
             self.w_q_norm = source.get(prefix + n["q_norm"]).float().contiguous()
             self.w_k_norm = source.get(prefix + n["k_norm"]).float().contiguous()
+        if self.learned_sink:
+            self.w_sink = source.get(prefix + n["sink"]).float().contiguous()
         if self.conv_taps:
             self.w_conv = torch.cat([source.get(prefix + n[k + "_conv"]).float() for k in kinds]).contiguous()
 
@@ -210,8 +227,9 @@ class Attention(Part):
         T = x.shape[0]
         width = 2 if ctx.act_dtype == torch.bfloat16 else 4
         q_dim, kv_dim = self.nh * self.hd, self.nkv * (self.hd + self.vd) // 2    # (kv_dim: the mean of a key's and a value's row)
-        with section("qkv", nbytes=width * (q_dim + 2 * kv_dim) * (self.hidden + T) + width * T * self.hidden,
-                     flops=2.0 * T * self.hidden * (q_dim + 2 * kv_dim)):
+        g_dim = self.nh * self.vd if self.has_gate else 0
+        with section("qkv", nbytes=width * (q_dim + 2 * kv_dim + g_dim) * (self.hidden + T) + width * T * self.hidden,
+                     flops=2.0 * T * self.hidden * (q_dim + 2 * kv_dim + g_dim)):
             qkv = ops.linear(x, self.w_qkv, ctx.act_dtype)
         slots = g.slot_mapping if cache.write else ctx.no_store_slots
         inv_freq = self.rotary.table(x.device) if self.rotary is not None else None
@@ -228,11 +246,14 @@ class Attention(Part):
             else:
                 q = ops.rope_kv(qkv, cache.k, cache.v, slots, ctx.positions, inv_freq, self.qk_norm_eps is not None,
                                 self.qk_norm_eps or 1e-6, self.q_temperature, self.nh, self.nkv, self.hd, layout,
-                                bias=self.b_qkv, vd=self.vd)
+                                bias=self.b_qkv, vd=self.vd, extra_columns=g_dim)
         with section("attention", nbytes=lambda: self._keys_held(ctx) * 2 * kv_dim * width + 2 * T * q_dim * width,
                      flops=lambda: 4.0 * self._keys_read(ctx) * q_dim):
             o = ops.attention(q, cache.k, cache.v, g, ctx, self.window_kind, self.window, self.scale, self.nh, self.nkv,
-                              self.hd, self.vd, softcap=self.softcap, sink=self.sink)
+                              self.hd, self.vd, softcap=self.softcap, sink=self.w_sink if self.learned_sink else self.sink)
+        if self.has_gate:
+            with section("output gate", nbytes=3 * width * T * g_dim):
+                o = ops.sigmoid_gate(o, qkv, qkv.shape[1] - g_dim)
         with section("o", nbytes=width * self.hidden * (q_dim + T) + width * T * q_dim, flops=2.0 * T * self.hidden * q_dim):
             out = ops.linear(o, self.w_o, ctx.act_dtype)
             return ops.add_bias(out, self.b_o) if self.b_o is not None else out

@@ -17,16 +17,25 @@ class PreNormBlock(Part):
     leaves its feed-forward output pending for the next block's first norm.  A feed-forward that
     has ``forward_from_stream(stream, norm, ctx)`` is handed the stream and the second norm instead
     of normalised rows (it must leave the stream as the norm would have).  Names of the four
-    parts in the weight file are arguments."""
+    parts in the weight file are arguments.  ``ffn`` None (with ``norm2`` None): a layer of a mixer
+    alone.  ``after``: a part with ``forward_on_stream(stream, ctx)`` that runs at the layer's end on
+    the residual sum itself (it adds the pending branch output first); its tensors lie under
+    ``names["after"]``."""
 
-    def __init__(self, norm1: Part, mixer: Part, norm2: Part, ffn: Part, names=None):
-        self.norm1, self.mixer, self.norm2, self.ffn = norm1, mixer, norm2, ffn
+    def __init__(self, norm1: Part, mixer: Part, norm2: Part = None, ffn: Part = None, names=None, after: Part = None):
+        if (norm2 is None) != (ffn is None):
+            raise ValueError("a feed-forward and its norm come together")
+        self.norm1, self.mixer, self.norm2, self.ffn, self.after_part = norm1, mixer, norm2, ffn, after
         self.names = dict(names or {"norm1": "input_layernorm.", "mixer": "self_attn.",
                                     "norm2": "post_attention_layernorm.", "ffn": "feed_forward."})
 
     def _children(self):
-        return ((self.names["norm1"], self.norm1), (self.names["mixer"], self.mixer),
-                (self.names["norm2"], self.norm2), (self.names["ffn"], self.ffn))
+        kids = [(self.names["norm1"], self.norm1), (self.names["mixer"], self.mixer)]
+        if self.ffn is not None:
+            kids += [(self.names["norm2"], self.norm2), (self.names["ffn"], self.ffn)]
+        if getattr(self, "after_part", None) is not None:
+            kids.append((self.names.get("after", "after."), self.after_part))
+        return tuple(kids)
 
     def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
         out: Dict[str, ParamSpec] = {}
@@ -61,9 +70,11 @@ class PreNormBlock(Part):
         from_stream = getattr(self.ffn, "forward_from_stream", None)
         if from_stream is not None:    # a feed-forward that may fuse the norm with work of its own
             stream.pending = from_stream(stream, self.norm2, ctx)
-        else:
+        elif self.ffn is not None:
             n = self.norm2.forward(stream, ctx.act_dtype)
             stream.pending = self.ffn.forward(n, ctx)
+        if self.after_part is not None:
+            self.after_part.forward_on_stream(stream, ctx)
 
 
 class PostNormBlock(PreNormBlock):

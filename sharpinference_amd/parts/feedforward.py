@@ -36,28 +36,48 @@ def _activation_code(name: str) -> int:
 class DenseSwiGLU(Part):
     """down( act(gate x) * (up x) ) (reference: src/SharpInference.Engine/ForwardPass.cs:2006-2015;
     silu(g) = g / (1 + exp(-g)), src/SharpInference.Cpu/SimdKernels.cs:4377-4408).  ``activation``
-    names the gate's function: "silu" (the reference's) or "gelu_tanh"."""
+    names the gate's function: "silu" (the reference's) or "gelu_tanh".  ``bias``: the three
+    products carry biases (``names`` + ``bias_suffix``), added in float: the gate's and the up
+    projection's inside the activation kernel, the down projection's by a row kernel.  ``names``:
+    the three matrices' names behind the part's prefix."""
 
-    def __init__(self, hidden: int, intermediate: int, activation: str = "silu"):
+    NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+
+    def __init__(self, hidden: int, intermediate: int, activation: str = "silu", bias: bool = False,
+                 names: Optional[Dict[str, str]] = None, bias_suffix: str = ".bias"):
         self.hidden, self.inter = int(hidden), int(intermediate)
         self.act = _activation_code(activation)
+        self.bias, self.bias_suffix = bool(bias), bias_suffix
+        self.names = {**self.NAMES, **(names or {})}
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_down: Optional[torch.Tensor] = None
+        self.b_gate_up: Optional[torch.Tensor] = None     # float32 [2 * inter]
+        self.b_down: Optional[torch.Tensor] = None        # float32 [hidden]
 
     def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
-        return {
-            prefix + "gate_proj.weight": ParamSpec((self.inter, self.hidden)),
-            prefix + "up_proj.weight": ParamSpec((self.inter, self.hidden)),
-            prefix + "down_proj.weight": ParamSpec((self.hidden, self.inter)),
+        n = self.names
+        out = {
+            prefix + n["gate"]: ParamSpec((self.inter, self.hidden)),
+            prefix + n["up"]: ParamSpec((self.inter, self.hidden)),
+            prefix + n["down"]: ParamSpec((self.hidden, self.inter)),
         }
+        if self.bias:
+            out.update({prefix + n["gate"] + self.bias_suffix: ParamSpec((self.inter,)),
+                        prefix + n["up"] + self.bias_suffix: ParamSpec((self.inter,)),
+                        prefix + n["down"] + self.bias_suffix: ParamSpec((self.hidden,))})
+        return out
 
     def load(self, prefix: str, source: TensorSource) -> None:
-        g = source.get(prefix + "gate_proj.weight")
-        u = source.get(prefix + "up_proj.weight")
+        n = self.names
+        g = source.get(prefix + n["gate"])
+        u = source.get(prefix + n["up"])
         # both also in the order the few-rows kernel streams them; the rows stay for prompt-sized steps
         self.w_gate_up = ops.pack_weight(_fuse_rows(g, u))
         del g, u
-        self.w_down = ops.pack_weight(source.get(prefix + "down_proj.weight"))
+        self.w_down = ops.pack_weight(source.get(prefix + n["down"]))
+        if self.bias:
+            self.b_gate_up = torch.cat([source.get(prefix + n[k] + self.bias_suffix).float() for k in ("gate", "up")]).contiguous()
+            self.b_down = source.get(prefix + n["down"] + self.bias_suffix).float().contiguous()
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         T = x.shape[0]
@@ -65,8 +85,9 @@ class DenseSwiGLU(Part):
         with section("dense feed-forward", nbytes=width * 3 * self.inter * self.hidden + width * T * (2 * self.hidden + 3 * self.inter),
                      flops=6.0 * T * self.inter * self.hidden):
             gu = ops.linear(x, self.w_gate_up, ctx.act_dtype)
-            act = ops.gated_act(gu, None, self.act)
-            return ops.linear(act, self.w_down, ctx.act_dtype)
+            act = ops.gated_act(gu, None, self.act, bias=self.b_gate_up)
+            out = ops.linear(act, self.w_down, ctx.act_dtype)
+            return ops.add_bias(out, self.b_down) if self.b_down is not None else out
 
 
 class DenseMLP(Part):

@@ -42,7 +42,8 @@ class DecoderModel(Part):
                  layer_prefix: str = "model.layers.", embed_name: str = "model.embed_tokens.weight",
                  norm_prefix: str = "model.norm.", head_name: str = "lm_head.weight", embedding_scale: float = 1.0,
                  logit_scale: float = 1.0, logit_softcap: Optional[float] = None,
-                 row_tables: Optional[Dict[str, int]] = None):
+                 row_tables: Optional[Dict[str, int]] = None, shared: Sequence[Part] = ()):
+        self.shared = list(shared)       # tensors that several parts read (parts/token_side.py:SharedTensor), loaded once
         self.row_tables: Dict[str, int] = dict(row_tables or {})      # name -> rows of a [rows, hidden] tensor
         self._row_table_f32: Dict[str, torch.Tensor] = {}
         self.vocab_size, self.hidden = int(vocab_size), int(hidden)
@@ -114,6 +115,8 @@ class DecoderModel(Part):
         for i, b in enumerate(self.blocks):
             out.update(b.param_specs(f"{self.layer_prefix}{i}."))
         out.update(self.final_norm.param_specs(self.norm_prefix))
+        for part in self.shared:
+            out.update(part.param_specs(""))
         for name, rows in self.row_tables.items():
             out[name] = ParamSpec((rows, self.hidden))
         if not self.tie_embeddings:
@@ -122,6 +125,8 @@ class DecoderModel(Part):
 
     def load_weights(self, source: TensorSource) -> None:
         self.embed = source.get(self.embed_name)
+        for part in self.shared:
+            part.load("", source)
         for i, b in enumerate(self.blocks):
             b.load(f"{self.layer_prefix}{i}.", source)
         self.final_norm.load(self.norm_prefix, source)

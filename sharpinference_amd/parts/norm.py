@@ -14,10 +14,12 @@ class RMSNorm(Part):
     """x * rsqrt(mean(x^2) + eps) * w, statistics in float
     (reference: src/SharpInference.Cpu/SimdKernels.cs:4209-4246; CUDA twin
     src/SharpInference.Cuda/CudaTextKernels.cs:199-224).  ``has_weight=False`` is the
-    weightless form (SimdKernels.cs:4252-4283)."""
+    weightless form (SimdKernels.cs:4252-4283).  ``weight_offset`` c: the stored weight lies around
+    zero and stands for c + w (the sum is formed once, in float, when the weight is loaded)."""
 
-    def __init__(self, dim: int, eps: float, has_weight: bool = True, name: str = "weight"):
+    def __init__(self, dim: int, eps: float, has_weight: bool = True, name: str = "weight", weight_offset: float = 0.0):
         self.dim, self.eps, self.has_weight = int(dim), float(eps), bool(has_weight)
+        self.weight_offset = float(weight_offset)
         self.name = name           # the weight's name behind the part's prefix ("" : the prefix is the name)
         self.weight: Optional[torch.Tensor] = None
         self._weight_f32: Optional[torch.Tensor] = None
@@ -28,6 +30,8 @@ class RMSNorm(Part):
     def load(self, prefix: str, source: TensorSource) -> None:
         if self.has_weight:
             self.weight = source.get(prefix + self.name)
+            if self.weight_offset:
+                self.weight = (self.weight.float() + self.weight_offset).contiguous()
             self._weight_f32 = None
 
     def add_normed(self, stream: ResidualStream, delta, out_dtype: Optional[torch.dtype]) -> None:
@@ -69,6 +73,13 @@ class RMSNorm(Part):
                 stream.pending = stream.pending_norm = None
                 return self.after(post, stream, delta, out_dtype)
             stream.settle()
+        if isinstance(stream.pending, ops.BranchSum):      # a scaled sum of branches: added in float, then the norm
+            if rows is None:
+                with section("norm", nbytes=stream.h.shape[0] * self.dim * (8 + 4 * len(stream.pending.xs))):
+                    ops.stream_add(stream.h, stream.pending)
+                stream.pending = None
+            else:
+                stream.pending = stream.pending.tensor()
         n = stream.h.shape[0] if rows is None else rows.shape[0]
         with section("norm", nbytes=n * self.dim * 12):
             out = ops.add_rmsnorm(stream.h, stream.pending, self.weight, self.eps, out_dtype, rows=rows,

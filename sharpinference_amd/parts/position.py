@@ -41,12 +41,20 @@ class YarnScaling:
     slow: float
 
 
+@dataclass(frozen=True)
+class LinearScaling:
+    """Position interpolation: every frequency divided by ``factor``."""
+
+    factor: float
+
+
 class Rotary(Part):
     """Rotary encoding: angle = pos * freq_i, freq_i = theta^(-2i/rotary_dim), i < rotary_dim/2,
     on the first ``rotary_dim`` elements of a head (all of it by default)
     (reference: src/SharpInference.Cpu/SimdKernels.cs:4591-4629, 4789-4811 for the interleaved
     pairing; the reference's other pairing and its partial width are IsNeoxRope and RopeDim,
-    src/SharpInference.Core/ModelGraph.cs:129-141).  ``scaling`` (llama3 rule) stretches the long
+    src/SharpInference.Core/ModelGraph.cs:129-141).  ``scaling``: a ``LinearScaling`` divides every
+    frequency by its factor; a ``WavelengthScaling`` (llama3 rule) stretches the long
     wavelengths: with wavelength L = 2*pi/freq and o the original context, L < o/high keeps freq,
     L > o/low divides it by factor, and between the two it is blended linearly in o/L.  The
     reference only consumes a precomputed divisor table
@@ -71,7 +79,9 @@ class Rotary(Part):
         for i in range(rd // 2):
             f = math.pow(self.theta, -2.0 * i / rd)
             s = self.scaling
-            if s is not None:
+            if isinstance(s, LinearScaling):
+                f = f / s.factor
+            elif s is not None:
                 wavelength = 2.0 * math.pi / f
                 lo_edge = s.original_max_position_embeddings / s.low_freq_factor
                 hi_edge = s.original_max_position_embeddings / s.high_freq_factor
