@@ -97,11 +97,8 @@ class Attention(Part):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads cannot share {num_kv_heads} kv heads")
         prep = bool(qk_norm_weights or values_from_keys or conv_taps)
-        if prep:
-            if head_dim % 2 or not 2 <= head_dim <= 256:
-                raise ValueError(f"head_dim {head_dim} is not taken: even sizes from 2 to 256")
-        elif head_dim % 16 or not 16 <= head_dim <= 256:
-            raise ValueError(f"head_dim {head_dim} is not taken: multiples of 16 from 16 to 256")
+        if head_dim % 2 or not 2 <= head_dim <= 256:      # (the rotation takes pairs; the attention kernels hold 256 elements)
+            raise ValueError(f"head_dim {head_dim} is not taken: even sizes from 2 to 256")
         if rotary is not None and rotary.head_dim != head_dim:
             raise ValueError("the rotary table's head_dim differs from the mixer's")
         if rotary is not None and rotary.pair_layout not in ("interleaved", "half"):
