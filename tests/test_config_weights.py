@@ -386,10 +386,10 @@ def test_prompts_as_text_or_ids(tmp_path):
 
 
 def test_a_head_size_no_kernel_takes_is_refused_when_the_model_is_built():
-    for hd in (272, 24):
-        cfg = load_config({**TINY_A, "head_dim": hd})
-        with pytest.raises(ValueError, match=f"head_dim {hd}"):
-            build_model(cfg)
+    cfg = load_config({**TINY_A, "head_dim": 272})
+    with pytest.raises(ValueError, match="head_dim 272"):
+        build_model(cfg)
+    build_model(load_config({**TINY_A, "head_dim": 24}))               # any even size up to 256 has a kernel
     with pytest.raises(ValueError, match="1025 experts"):
         build_model(load_config({**TINY_A, "num_local_experts": 1025}))
 
