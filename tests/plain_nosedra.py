@@ -19,6 +19,19 @@ import torch
 DENOMINATOR_FLOOR = 1e-6      # added to the matrix memory's normaliser
 
 
+def _same(x: torch.Tensor) -> torch.Tensor:
+    return x
+
+
+def store_bf16(x: torch.Tensor) -> torch.Tensor:
+    """x rounded to bfloat16 and widened again: what a tensor kept in 16 bits loses.  Handed to the
+    functions below as ``store``, it is applied where a 16-bit engine may keep a tensor (the outputs
+    of matrix products, of norms, of activations and of the attention), and nowhere in what the
+    design computes in 32 bits (scores and softmax, gates and decays, states, norms' statistics, the
+    residual sum): the difference to the exact run shows how far rounding alone moves a result."""
+    return x.to(torch.bfloat16).to(x.dtype)
+
+
 def read_config(model_dir: str) -> dict:
     with open(os.path.join(model_dir, "config.json")) as f:
         return json.load(f)
@@ -129,19 +142,20 @@ def sink_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: flo
     return out
 
 
-def left_mixer(h: torch.Tensor, positions: torch.Tensor, p: Dict[str, torch.Tensor], pre: str, m: dict, eps: float) -> torch.Tensor:
+def left_mixer(h: torch.Tensor, positions: torch.Tensor, p: Dict[str, torch.Tensor], pre: str, m: dict, eps: float,
+               store=_same) -> torch.Tensor:
     T = h.shape[0]
     H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = (h @ p[pre + "q"].T).view(T, H, d)
-    k = (h @ p[pre + "k"].T).view(T, G, d)
-    v = (h @ p[pre + "v"].T).view(T, G, e)
+    q = store(h @ p[pre + "q"].T).view(T, H, d)
+    k = store(h @ p[pre + "k"].T).view(T, G, d)
+    v = store(h @ p[pre + "v"].T).view(T, G, e)
     if m.get("rot"):
         f = frequencies(m["rot"])
         q, k = rotate_halves(q, positions, f), rotate_halves(k, positions, f)
-    q, k = unit_rms(q, eps), unit_rms(k, eps)
-    o = sink_attention(q, k, v, m["scale"], p[pre + "sink"]).reshape(T, H * e)
-    o = o * torch.sigmoid(h @ p[pre + "g"].T)
-    return o @ p[pre + "o"].T
+    q, k = store(unit_rms(q, eps)), store(unit_rms(k, eps))
+    o = store(sink_attention(q, k, v, m["scale"], p[pre + "sink"]).reshape(T, H * e))
+    o = store(o * torch.sigmoid(store(h @ p[pre + "g"].T)))
+    return store(o @ p[pre + "o"].T)
 
 
 # ----------------------------------------------------------------------------
@@ -168,22 +182,23 @@ def matrix_memory(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, log_i: torc
     return out
 
 
-def right_mixer(h: torch.Tensor, p: Dict[str, torch.Tensor], pre: str, m: dict, eps: float) -> torch.Tensor:
+def right_mixer(h: torch.Tensor, p: Dict[str, torch.Tensor], pre: str, m: dict, eps: float, store=_same) -> torch.Tensor:
     T = h.shape[0]
     H, d, e, cap = m["heads"], m["dim"], m["vdim"], float(m["gate_cap"])
-    q = (h @ p[pre + "q"].T).view(T, H, d) * d ** -0.5
-    k = (h @ p[pre + "k"].T).view(T, H, d)
-    v = (h @ p[pre + "v"].T).view(T, H, e)
+    q = store(h @ p[pre + "q"].T).view(T, H, d) * d ** -0.5
+    k = store(h @ p[pre + "k"].T).view(T, H, d)
+    v = store(h @ p[pre + "v"].T).view(T, H, e)
     log_i = capped(h @ p[pre + "i"].T + p[pre + "i.b"], cap)
     log_f = log_sigmoid(capped(h @ p[pre + "f"].T + p[pre + "f.b"], cap))
     o = unit_rms(matrix_memory(q, k, v, log_i, log_f), eps).reshape(T, H * e)
-    o = o * p[pre + "norm"] * torch.sigmoid(h @ p[pre + "g"].T)
-    return o @ p[pre + "o"].T
+    o = store(o * p[pre + "norm"] * torch.sigmoid(store(h @ p[pre + "g"].T)))
+    return store(o @ p[pre + "o"].T)
 
 
-def parallel_mixer(h: torch.Tensor, positions: torch.Tensor, p: Dict[str, torch.Tensor], pre: str, m: dict, eps: float) -> torch.Tensor:
-    return m["left_scale"] * left_mixer(h, positions, p, pre + "left.", m["left"], eps) + \
-        m["right_scale"] * right_mixer(h, p, pre + "right.", m["right"], eps)
+def parallel_mixer(h: torch.Tensor, positions: torch.Tensor, p: Dict[str, torch.Tensor], pre: str, m: dict, eps: float,
+                   store=_same) -> torch.Tensor:
+    return m["left_scale"] * left_mixer(h, positions, p, pre + "left.", m["left"], eps, store) + \
+        m["right_scale"] * right_mixer(h, p, pre + "right.", m["right"], eps, store)
 
 
 # ----------------------------------------------------------------------------
@@ -205,67 +220,69 @@ def state_space_scan(x: torch.Tensor, B: torch.Tensor, C: torch.Tensor, dt: torc
     return y
 
 
-def state_space_mixer(h: torch.Tensor, p: Dict[str, torch.Tensor], pre: str, m: dict, eps: float) -> torch.Tensor:
+def state_space_mixer(h: torch.Tensor, p: Dict[str, torch.Tensor], pre: str, m: dict, eps: float, store=_same) -> torch.Tensor:
     T = h.shape[0]
     H, e, d, G, parts = m["heads"], m["vdim"], m["state"], m["groups"], m["norm_groups"]
     inner = H * e
     u = h @ p[pre + "in"].T
-    z, xBC, dt = u[:, :inner], u[:, inner:2 * inner + 2 * G * d], u[:, 2 * inner + 2 * G * d:]
-    xBC = silu(biased_convolution(xBC, p[pre + "conv"], p[pre + "conv.b"]))
+    z, xBC, dt = store(u[:, :inner]), store(u[:, inner:2 * inner + 2 * G * d]), u[:, 2 * inner + 2 * G * d:]
+    xBC = store(silu(biased_convolution(xBC, p[pre + "conv"], p[pre + "conv.b"])))
     x = xBC[:, :inner].view(T, H, e)
     B = xBC[:, inner:inner + G * d].view(T, G, d)
     C = xBC[:, inner + G * d:].view(T, G, d)
     dt = softplus(dt + p[pre + "dt_bias"])
     y = state_space_scan(x, B, C, dt, p[pre + "A_log"], p[pre + "D"]).reshape(T, inner)
     y = y * silu(z)
-    y = unit_rms(y.view(T, parts, inner // parts), eps).reshape(T, inner) * p[pre + "norm"]
-    return y @ p[pre + "o"].T
+    y = store(unit_rms(y.view(T, parts, inner // parts), eps).reshape(T, inner) * p[pre + "norm"])
+    return store(y @ p[pre + "o"].T)
 
 
 # ----------------------------------------------------------------------------
 # feed-forward, the per-layer token input, layers, the model
 # ----------------------------------------------------------------------------
-def gated_feed_forward(h: torch.Tensor, p: Dict[str, torch.Tensor], pre: str) -> torch.Tensor:
-    gate = gelu_tanh(h @ p[pre + "gate"].T + p[pre + "gate.b"])
-    up = h @ p[pre + "up"].T + p[pre + "up.b"]
-    return (gate * up) @ p[pre + "down"].T + p[pre + "down.b"]
+def gated_feed_forward(h: torch.Tensor, p: Dict[str, torch.Tensor], pre: str, store=_same) -> torch.Tensor:
+    gate = gelu_tanh(store(h @ p[pre + "gate"].T) + p[pre + "gate.b"])
+    up = store(h @ p[pre + "up"].T) + p[pre + "up.b"]
+    return store(store(store(gate * up) @ p[pre + "down"].T) + p[pre + "down.b"])
 
 
-def token_input(x: torch.Tensor, tokens: torch.Tensor, p: Dict[str, torch.Tensor], i: int, dim: int, eps: float) -> torch.Tensor:
+def token_input(x: torch.Tensor, tokens: torch.Tensor, p: Dict[str, torch.Tensor], i: int, dim: int, eps: float, store=_same) -> torch.Tensor:
     """What layer i adds at its end: its slice of the side table's row of each token, gated by the stream."""
     pre = f"l{i}.side."
     e = p["side.embed"][tokens][:, i * dim:(i + 1) * dim]
-    y = (gelu_tanh(x @ p[pre + "gate"].T) * e) @ p[pre + "proj"].T
+    y = store(store(gelu_tanh(store(store(x) @ p[pre + "gate"].T)) * e) @ p[pre + "proj"].T)
     return unit_rms(y, eps) * p[pre + "norm"]
 
 
-def run_layer(cfg: dict, x: torch.Tensor, tokens: torch.Tensor, positions: torch.Tensor, p: Dict[str, torch.Tensor], i: int) -> torch.Tensor:
+def run_layer(cfg: dict, x: torch.Tensor, tokens: torch.Tensor, positions: torch.Tensor, p: Dict[str, torch.Tensor], i: int,
+              store=_same) -> torch.Tensor:
     layer, eps = cfg["layers"][i], cfg["norm"]["eps"]
     pre = f"l{i}."
-    h = offset_norm(x, p[pre + "norm1"], eps)
+    h = store(offset_norm(x, p[pre + "norm1"], eps))
     if layer["type"] == "parallel":
-        x = x + parallel_mixer(h, positions, p, pre + "mix.", layer["mixer"], eps)
+        x = x + parallel_mixer(h, positions, p, pre + "mix.", layer["mixer"], eps, store)
     elif layer["type"] == "mamba2":
-        x = x + state_space_mixer(h, p, pre + "mix.", layer["mixer"], eps)
+        x = x + state_space_mixer(h, p, pre + "mix.", layer["mixer"], eps, store)
     else:
         raise ValueError(f"layer type {layer['type']!r}")
     if layer.get("mlp") is not None:
-        x = x + gated_feed_forward(offset_norm(x, p[pre + "norm2"], eps), p, pre + "mlp.")
+        x = x + gated_feed_forward(store(offset_norm(x, p[pre + "norm2"], eps)), p, pre + "mlp.", store)
     if cfg.get("token_side"):
-        x = x + token_input(x, tokens, p, i, cfg["token_side"]["dim"], eps)
+        x = x + token_input(x, tokens, p, i, cfg["token_side"]["dim"], eps, store)
     return x
 
 
-def forward(cfg: dict, p: Dict[str, torch.Tensor], tokens: Sequence[int], layers_out: Optional[list] = None) -> torch.Tensor:
-    """Logits [T, vocab] of a whole sequence; ``layers_out`` receives the stream after every layer."""
+def forward(cfg: dict, p: Dict[str, torch.Tensor], tokens: Sequence[int], layers_out: Optional[list] = None, store=_same) -> torch.Tensor:
+    """Logits [T, vocab] of a whole sequence; ``layers_out`` receives the stream after every layer;
+    ``store`` (see ``store_bf16``) rounds what a 16-bit engine may keep in 16 bits."""
     tok = torch.as_tensor(list(tokens), dtype=torch.int64)
     positions = torch.arange(tok.shape[0])
     x = p["embed"][tok]
     for i in range(len(cfg["layers"])):
-        x = run_layer(cfg, x, tok, positions, p, i)
+        x = run_layer(cfg, x, tok, positions, p, i, store)
         if layers_out is not None:
             layers_out.append(x.clone())
-    logits = offset_norm(x, p["final.norm"], cfg["norm"]["eps"]) @ p["head"].T
+    logits = store(offset_norm(x, p["final.norm"], cfg["norm"]["eps"])) @ p["head"].T
     cap = cfg.get("logit_softcap")
     return capped(logits, float(cap)) if cap else logits
 
