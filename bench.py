@@ -14,7 +14,9 @@ prompts read in 4,096-token portions beside decoding requests) and print a JSON 
 ``--shape kuvonex`` runs Kuvonex layers (latent attention, routed experts in groups) at two sizes,
 each beside Llama 4 layers of the same width, heads and experts, with the kernel-class tables of both;
 ``--shape pazatar`` does the same for Pazatar layers (attention that norms before it rotates, gated linear
-attention beside it, dense feed-forwards) beside Llama 4 layers with dense feed-forwards.
+attention beside it, dense feed-forwards) beside Llama 4 layers with dense feed-forwards;
+``--shape nosedra`` runs Nosedra layers (attention with a learned sink beside a matrix memory with exponential
+gates, state-space layers) beside Pazatar layers of the same sizes.
 """
 from __future__ import annotations
 
@@ -573,8 +575,9 @@ def pazatar_config(z: dict) -> dict:
             "rot": {"base": 20000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 2048}}}
     right = {"heads": z["heads"], "dim": 128, "vdim": 128, "tau": 16.0, "decay_rank": z["decay_rank"]}
     mlp = {"kind": "dense", "ff": z["ff"]}
-    layers = [{"type": "attention", "mixer": attention, "mlp": mlp} if i % 2 == 0 else
-              {"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp} for i in range(z["layers"])]
+    kinds = z.get("kinds") or ["attention" if i % 2 == 0 else "parallel" for i in range(z["layers"])]
+    layers = [{"type": "attention", "mixer": attention, "mlp": mlp} if kind == "attention" else
+              {"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp} for kind in kinds]
     return {"architecture": "Pazatar", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-5}, "layers": layers,
             "loop": {"start": 0, "stop": z["layers"], "times": 1}}
 
@@ -608,6 +611,53 @@ def run_pazatar(args) -> int:
     return 0
 
 
+# ---------------------------------------------------------------------------
+# Nosedra beside Pazatar at equal sizes
+# ---------------------------------------------------------------------------
+# width, layers (three parallel layers and a state-space layer in third place), attention heads of 128 over kv heads,
+# the matrix memory's heads of 128 key and 128 value channels, the state space's heads of 64 values over a state of
+# 128 in 8 groups (twice the width in all) behind four taps, feed-forward width, the token input's width, vocabulary
+NOSEDRA_SIZES = {
+    "w2048": dict(width=2048, layers=4, heads=16, kv_heads=4, ff=8192, vocab=32000, side=256, chunk=1024, decay_rank=64),
+    "w4096": dict(width=4096, layers=4, heads=32, kv_heads=8, ff=14336, vocab=32000, side=256, chunk=1024, decay_rank=128),
+}
+NOSEDRA_KINDS = ["parallel", "parallel", "mamba2", "parallel"]
+
+
+def nosedra_config(z: dict) -> dict:
+    left = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+            "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 2.0}}}
+    right = {"heads": z["heads"], "dim": 128, "vdim": 128, "gate_cap": 15.0}
+    space = {"heads": 2 * z["width"] // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    layers = [{"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}, "mlp": mlp}
+              if kind == "parallel" else {"type": "mamba2", "mixer": space, "mlp": mlp} for kind in NOSEDRA_KINDS[:z["layers"]]]
+    return {"architecture": "Nosedra", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-5},
+            "token_side": {"dim": z["side"]}, "logit_softcap": 30.0, "layers": layers}
+
+
+def pazatar_like_nosedra(z: dict) -> dict:
+    """Pazatar layers of the same width, heads and feed-forward width: a parallel layer (attention beside gated
+    linear attention) where Nosedra has one, an attention layer where it has its state space."""
+    return pazatar_config(dict(z, kinds=["parallel" if kind == "parallel" else "attention" for kind in NOSEDRA_KINDS[:z["layers"]]]))
+
+
+def run_nosedra(args) -> int:
+    """Prefill of one 2,048-token prompt and decode at batch 8 and 64 for the Nosedra design at two sizes
+    (random weights), each beside Pazatar layers of the same width, heads and feed-forward width, with the
+    per-kernel-class tables of one prefill and one decode step of both."""
+    rows, P, steps, warm = _beside(args, NOSEDRA_SIZES, (("nosedra", nosedra_config), ("pazatar", pazatar_like_nosedra)))
+    k0 = rows[0]
+    out = {"metric": "decode tok/s at batch 8 (Nosedra, width 2048, 4 layers, 2,048-token prompts)", "value": k0["decode_b8_tok_s"],
+           "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": k0["decode_b8_ms_per_step"],
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"model": "nosedra-random beside pazatar-random at equal sizes", "global_batch": 8, "seq_len": CONTEXT,
+                      "parallelism": "single-gpu", "prompt_len": P, "sizes": NOSEDRA_SIZES},
+           "rows": rows}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -621,9 +671,9 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel instead of replaying a HIP graph")
     ap.add_argument("--no-peaks", action="store_true", help="skip the two measuring kernels (pure read, matrix-core loop)")
     ap.add_argument("--profile", action="store_true", help="also print ms / bytes / GB/s per kernel class of one prefill and one decode step")
-    ap.add_argument("--shape", default="scout", choices=["scout", "maverick8", "long16", "kuvonex", "pazatar"],
+    ap.add_argument("--shape", default="scout", choices=["scout", "maverick8", "long16", "kuvonex", "pazatar", "nosedra"],
                     help="scout: the headline run; maverick8 / long16: two other workloads; kuvonex / pazatar: that design beside "
-                         "Llama 4 layers of equal size; each prints a JSON line of its own")
+                         "Llama 4 layers of equal size; nosedra: that design beside Pazatar layers of equal size; each prints a JSON line of its own")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path (N=1 only)")
@@ -636,6 +686,8 @@ def main() -> int:
         return run_kuvonex(args)
     if args.shape == "pazatar":
         return run_pazatar(args)
+    if args.shape == "nosedra":
+        return run_nosedra(args)
 
     import torch  # noqa: F401
 

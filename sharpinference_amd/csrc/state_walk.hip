@@ -22,9 +22,20 @@
 // lanes' order (row g RPL + r of column j at r 64 + 8 g + j), and, for the exponential gates, DKP
 // floats of n and the maximum m (each slice its own copy: the blocks of a head do not wait for
 // each other).
+//
+// A long entry alone in its step would leave most of the chip idle.  Since a_t is one number per head,
+// a stretch of tokens acts on the state as S -> D S + L with D the product of its decays and L what
+// the stretch makes of a zero state, so the entry is cut into segments that are walked side by side:
+// WALK_LOCAL walks every segment but an entry's last from nothing (for the exponential gates the
+// maximum starts at minus infinity: the first token then enters with weight 1) and keeps L, its
+// maximum and the summed logarithms of the decays; a short kernel turns these into the segments' true
+// start states one after the other (for the gates, with m' = max(F + m, m_L):
+// S' = exp(F + m - m') S + exp(m_L - m') L); WALK_FINAL walks every segment from its start state,
+// writes the outputs, and the entry's last segment leaves the new state in the slot.
 #include "common.h"
 
 enum : int { WALK_EXP_GATES = 0, WALK_STATE_SPACE = 1 };
+enum : int { WALK_WHOLE = 0, WALK_LOCAL = 1, WALK_FINAL = 2 };
 constexpr int kWalkCols = 8;       // value columns of a block
 constexpr int kWalkChunk = 16;     // tokens staged at a time
 constexpr float kWalkFloor = 1e-6f;
@@ -43,6 +54,13 @@ SHARPI_EXPORT int sharpi_state_walk_slice_floats(int dk, int mode) {
 __device__ __forceinline__ float softplus_f32(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
 __device__ __forceinline__ float log_sigmoid_f32(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
 
+// 16 bytes of a row as floats
+__device__ __forceinline__ void load16(const float* p, float* v) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+}
+__device__ __forceinline__ void load16(const bf16_t* p, float* v) { load8(p, v); }
+
 // where row `row` (= g RPL + r) of a staged q or k vector lies in LDS: four rows of a lane together,
 // the eight row groups side by side (a lane reads float4s, the wave 32 consecutive words)
 template <int RPL>
@@ -51,39 +69,62 @@ __device__ __forceinline__ int staged_at(int row) {
   return ((r >> 2) * 8 + g) * 4 + (r & 3);
 }
 
-template <typename T, int RPL, int MODE>
+template <typename T, int RPL, int MODE, int PHASE>
 __global__ __launch_bounds__(kWave) void state_walk_kernel(
     const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off, int heads_per_group,
     const float* __restrict__ gates, int gate_stride, const float* __restrict__ p0, const float* __restrict__ p1,
     const float* __restrict__ p2, float cap, float q_scale, float* __restrict__ state,
     const int* __restrict__ state_slots, const int* __restrict__ cu_tokens, float* __restrict__ out, int nh, int dk,
-    int dv, int ncb) {
+    int dv, int ncb, int vec, const int* __restrict__ segs, float* __restrict__ seg_local,
+    const float* __restrict__ seg_start, float* __restrict__ seg_decay) {
   constexpr int DKP = RPL * 8;
+  constexpr int V = 16 / (int)sizeof(T);            // elements of a 16-byte load
   __shared__ __attribute__((aligned(16))) float q_s[kWalkChunk][DKP];
   __shared__ __attribute__((aligned(16))) float k_s[kWalkChunk][DKP];
   __shared__ float v_s[kWalkChunk][kWalkCols];
   __shared__ float a_s[kWalkChunk], b_s[kWalkChunk], e_s[kWalkChunk];
-  const int cb = blockIdx.x, h = blockIdx.y, e = blockIdx.z;
+  const int cb = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x, g = lane >> 3, j = lane & 7;
-  const int t_first = cu_tokens[e], t_end = cu_tokens[e + 1];
-  if (t_end <= t_first) return;
   const int slice = walk_slice_floats(DKP, MODE);
-  float* st = state + (((size_t)state_slots[e] * nh + h) * ncb + cb) * slice;
+  int e, t_first, t_end;
+  bool last = true;
+  if (PHASE == WALK_WHOLE) {
+    e = blockIdx.z;
+    t_first = cu_tokens[e];
+    t_end = cu_tokens[e + 1];
+  } else {
+    const int* sg = segs + 4 * blockIdx.z;
+    e = sg[0];
+    t_first = sg[1];
+    t_end = t_first + sg[2];
+    last = sg[3] != 0;
+    if (PHASE == WALK_LOCAL && last) return;        // nobody starts from what an entry's last segment makes
+  }
+  if (t_end <= t_first) return;
+  const size_t seg_at = (((size_t)blockIdx.z * nh + h) * ncb + cb) * slice;
+  float* st = state + (((size_t)state_slots[e] * nh + h) * ncb + cb) * slice;      // the request's slot
+  const float* from = PHASE == WALK_FINAL ? seg_start + seg_at : st;
   const int c = cb * kWalkCols + j;
   const int qk_head = h / heads_per_group;
 
   float S[RPL], n[RPL];
+  float m_run = 0.f, log_decay = 0.f;
+  if (PHASE == WALK_LOCAL) {
 #pragma unroll
-  for (int r = 0; r < RPL; ++r) S[r] = st[r * 64 + lane];
-  float m_run = 0.f;
-  if (MODE == WALK_EXP_GATES) {
-    const float4* nsrc = reinterpret_cast<const float4*>(st + RPL * 64);
+    for (int r = 0; r < RPL; ++r) S[r] = 0.f, n[r] = 0.f;
+    m_run = -INFINITY;
+  } else {
 #pragma unroll
-    for (int r4 = 0; r4 < RPL / 4; ++r4) {
-      const float4 x = nsrc[r4 * 8 + g];
-      n[r4 * 4] = x.x; n[r4 * 4 + 1] = x.y; n[r4 * 4 + 2] = x.z; n[r4 * 4 + 3] = x.w;
+    for (int r = 0; r < RPL; ++r) S[r] = from[r * 64 + lane];
+    if (MODE == WALK_EXP_GATES) {
+      const float4* nsrc = reinterpret_cast<const float4*>(from + RPL * 64);
+#pragma unroll
+      for (int r4 = 0; r4 < RPL / 4; ++r4) {
+        const float4 x = nsrc[r4 * 8 + g];
+        n[r4 * 4] = x.x; n[r4 * 4 + 1] = x.y; n[r4 * 4 + 2] = x.z; n[r4 * 4 + 3] = x.w;
+      }
+      m_run = from[RPL * 64 + DKP];
     }
-    m_run = st[RPL * 64 + DKP];
   }
   float par0 = 0.f, par1 = 0.f, par2 = 0.f;     // the head's constants
   if (MODE == WALK_EXP_GATES) {
@@ -99,6 +140,26 @@ __global__ __launch_bounds__(kWave) void state_walk_kernel(
     const int nt = min(kWalkChunk, t_end - t0);
     __syncthreads();
     // stage q and k (floats, the lanes' order), v, and the tokens' gates
+    if (vec) {                                       // 16-byte loads: every head's q and k begin on a 16-byte border
+      constexpr int VPR = DKP / V;                   // loads of a row
+      for (int idx = lane; idx < kWalkChunk * VPR; idx += kWave) {
+        const int tt = idx / VPR, row0 = (idx % VPR) * V;
+        float qv[V], kv[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) qv[i] = 0.f, kv[i] = 0.f;
+        if (tt < nt && row0 < dk) {
+          const T* base = proj + (size_t)(t0 + tt) * stride + (size_t)qk_head * dk + row0;
+          load16(base + q_off, qv);
+          load16(base + k_off, kv);
+        }
+#pragma unroll
+        for (int i = 0; i < V; i += 4) {             // four rows of a lane lie together
+          const int at = staged_at<RPL>(row0 + i);
+          *reinterpret_cast<float4*>(&q_s[tt][at]) = make_float4(qv[i] * q_scale, qv[i + 1] * q_scale, qv[i + 2] * q_scale, qv[i + 3] * q_scale);
+          *reinterpret_cast<float4*>(&k_s[tt][at]) = make_float4(kv[i], kv[i + 1], kv[i + 2], kv[i + 3]);
+        }
+      }
+    } else
     for (int idx = lane; idx < kWalkChunk * DKP; idx += kWave) {
       const int tt = idx / DKP, row = idx % DKP;
       float qv = 0.f, kv = 0.f;
@@ -146,10 +207,20 @@ __global__ __launch_bounds__(kWave) void state_walk_kernel(
           e_s[lane] = expf(-m_t);
         }
         m_run = __shfl(m_t, nt - 1, kWave);
-      } else if (live) {
-        const float dt = softplus_f32(grow[h] + par0);
-        a_s[lane] = expf(par1 * dt);
-        b_s[lane] = dt;
+        if (PHASE == WALK_LOCAL) log_decay += __shfl(F, nt - 1, kWave);
+      } else {
+        float la = 0.f;
+        if (live) {
+          const float dt = softplus_f32(grow[h] + par0);
+          la = par1 * dt;
+          a_s[lane] = expf(la);
+          b_s[lane] = dt;
+        }
+        if (PHASE == WALK_LOCAL) {
+#pragma unroll
+          for (int off = 1; off < kWalkChunk; off <<= 1) la += __shfl_xor(la, off, kWave);
+          log_decay += la;
+        }
       }
     }
     __syncthreads();
@@ -168,13 +239,14 @@ __global__ __launch_bounds__(kWave) void state_walk_kernel(
         for (int i = 0; i < 4; ++i) {
           const int r = r4 * 4 + i;
           S[r] = fmaf(kr[i], bv, a * S[r]);
-          acc = fmaf(S[r], qr[i], acc);
+          if (PHASE != WALK_LOCAL) acc = fmaf(S[r], qr[i], acc);
           if (MODE == WALK_EXP_GATES) {
             n[r] = fmaf(kr[i], b, a * n[r]);
-            nq = fmaf(n[r], qr[i], nq);
+            if (PHASE != WALK_LOCAL) nq = fmaf(n[r], qr[i], nq);
           }
         }
       }
+      if (PHASE == WALK_LOCAL) continue;
       acc += __shfl_xor(acc, 8, kWave);
       acc += __shfl_xor(acc, 16, kWave);
       acc += __shfl_xor(acc, 32, kWave);
@@ -190,6 +262,11 @@ __global__ __launch_bounds__(kWave) void state_walk_kernel(
       if (g == 0 && c < dv) out[(size_t)(t0 + tt) * nh * dv + (size_t)h * dv + c] = y;
     }
   }
+  if (PHASE == WALK_FINAL && !last) return;
+  if (PHASE == WALK_LOCAL) {
+    st = seg_local + seg_at;
+    if (cb == 0 && lane == 0) seg_decay[(size_t)blockIdx.z * nh + h] = log_decay;
+  }
 #pragma unroll
   for (int r = 0; r < RPL; ++r) st[r * 64 + lane] = S[r];
   if (MODE == WALK_EXP_GATES) {
@@ -202,26 +279,108 @@ __global__ __launch_bounds__(kWave) void state_walk_kernel(
   }
 }
 
-template <typename T, int MODE>
-static int launch_state_walk(const void* proj, int stride, int q_off, int k_off, int v_off, int heads_per_group,
-                             const float* gates, int gate_stride, const float* p0, const float* p1, const float* p2,
-                             float cap, float q_scale, float* state, const int* state_slots, const int* cu_tokens,
-                             float* out, int n_entries, int nh, int dk, int dv, hipStream_t stream) {
-  const int ncb = ceil_div(dv, kWalkCols);
-  dim3 grid(ncb, nh, n_entries);
-#define WALK(RPL)                                                                                                      \
-  state_walk_kernel<T, RPL, MODE><<<grid, kWave, 0, stream>>>((const T*)proj, stride, q_off, k_off, v_off,             \
-                                                              heads_per_group, gates, gate_stride, p0, p1, p2, cap,    \
-                                                              q_scale, state, state_slots, cu_tokens, out, nh, dk, dv, \
-                                                              ncb)
-  if (dk <= 32) WALK(4);
-  else if (dk <= 64) WALK(8);
-  else if (dk <= 128) WALK(16);
-  else if (dk <= 256) WALK(32);
-  else return SHARPI_ERR_ARG;
-#undef WALK
+// The segments' start states, one entry's after the other: start(first) = the slot's state, start(s + 1) =
+// what segment s makes of start(s).  A block = (8 value columns, head, entry); a lane moves the floats
+// lane, lane + 64, .. of the slice (S and, for the gates, n; each lane reads only what it wrote).
+template <int MODE>
+__global__ __launch_bounds__(kWave) void state_walk_combine_kernel(
+    const float* __restrict__ state, const int* __restrict__ state_slots, const int* __restrict__ ent_segs,
+    const float* __restrict__ seg_local, float* __restrict__ seg_start, const float* __restrict__ seg_decay, int nh,
+    int ncb, int dkp) {
+  const int cb = blockIdx.x, h = blockIdx.y, e = blockIdx.z, lane = threadIdx.x;
+  const int first = ent_segs[2 * e], count = ent_segs[2 * e + 1];
+  if (count <= 0) return;
+  const int slice = walk_slice_floats(dkp, MODE);
+  const int moved = (dkp / 8) * 64 + (MODE == WALK_EXP_GATES ? dkp : 0);     // S and n
+  const float* slot = state + (((size_t)state_slots[e] * nh + h) * ncb + cb) * slice;
+  float* cur = seg_start + (((size_t)first * nh + h) * ncb + cb) * slice;
+  for (int i = lane; i < moved; i += kWave) cur[i] = slot[i];
+  float m = 0.f;
+  if (MODE == WALK_EXP_GATES) {
+    m = slot[moved];
+    if (lane == 0) cur[moved] = m;
+  }
+  for (int s = first; s + 1 < first + count; ++s) {
+    const size_t at = (((size_t)s * nh + h) * ncb + cb) * slice;
+    const float* loc = seg_local + at;
+    float* next = seg_start + at + (size_t)nh * ncb * slice;
+    const float F = seg_decay[(size_t)s * nh + h];
+    float wa, wb = 1.f;
+    if (MODE == WALK_EXP_GATES) {
+      const float m_loc = loc[moved];
+      const float m_new = fmaxf(F + m, m_loc);
+      wa = expf(F + m - m_new);
+      wb = expf(m_loc - m_new);
+      m = m_new;
+      if (lane == 0) next[moved] = m;
+    } else {
+      wa = expf(F);
+    }
+    for (int i = lane; i < moved; i += kWave) next[i] = fmaf(wa, cur[i], wb * loc[i]);
+    cur = next;
+  }
+}
+
+struct WalkArgs {
+  const void* proj; int stride, q_off, k_off, v_off, heads_per_group;
+  const float* gates; int gate_stride; const float *p0, *p1, *p2;
+  float cap, q_scale; float* state; const int *state_slots, *cu_tokens; float* out;
+  int n_entries, nh, dk, dv;
+  const int *segs, *ent_segs; int n_segs; float *seg_local, *seg_start, *seg_decay;
+};
+
+template <typename T, int RPL, int MODE, int PHASE>
+static void launch_walk_phase(const WalkArgs& a, int ncb, int vec, hipStream_t stream) {
+  dim3 grid(ncb, a.nh, PHASE == WALK_WHOLE ? a.n_entries : a.n_segs);
+  state_walk_kernel<T, RPL, MODE, PHASE><<<grid, kWave, 0, stream>>>(
+      (const T*)a.proj, a.stride, a.q_off, a.k_off, a.v_off, a.heads_per_group, a.gates, a.gate_stride, a.p0, a.p1, a.p2,
+      a.cap, a.q_scale, a.state, a.state_slots, a.cu_tokens, a.out, a.nh, a.dk, a.dv, ncb, vec, a.segs, a.seg_local,
+      a.seg_start, a.seg_decay);
+}
+
+template <typename T, int RPL, int MODE>
+static int launch_walk_rpl(const WalkArgs& a, int ncb, int vec, hipStream_t stream) {
+  if (!a.segs) {
+    launch_walk_phase<T, RPL, MODE, WALK_WHOLE>(a, ncb, vec, stream);
+    SHARPI_CHECK_LAUNCH();
+    return SHARPI_OK;
+  }
+  launch_walk_phase<T, RPL, MODE, WALK_LOCAL>(a, ncb, vec, stream);
+  SHARPI_CHECK_LAUNCH();
+  state_walk_combine_kernel<MODE><<<dim3(ncb, a.nh, a.n_entries), kWave, 0, stream>>>(
+      a.state, a.state_slots, a.ent_segs, a.seg_local, a.seg_start, a.seg_decay, a.nh, ncb, RPL * 8);
+  SHARPI_CHECK_LAUNCH();
+  launch_walk_phase<T, RPL, MODE, WALK_FINAL>(a, ncb, vec, stream);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
+}
+
+template <typename T, int MODE>
+static int launch_state_walk(const WalkArgs& a, hipStream_t stream) {
+  const int ncb = ceil_div(a.dv, kWalkCols);
+  constexpr int V = 16 / (int)sizeof(T);
+  const int vec = a.dk % V == 0 && a.stride % V == 0 && a.q_off % V == 0 && a.k_off % V == 0 &&
+                  reinterpret_cast<uintptr_t>(a.proj) % 16 == 0;
+  if (a.dk <= 32) return launch_walk_rpl<T, 4, MODE>(a, ncb, vec, stream);
+  if (a.dk <= 64) return launch_walk_rpl<T, 8, MODE>(a, ncb, vec, stream);
+  if (a.dk <= 128) return launch_walk_rpl<T, 16, MODE>(a, ncb, vec, stream);
+  if (a.dk <= 256) return launch_walk_rpl<T, 32, MODE>(a, ncb, vec, stream);
+  return SHARPI_ERR_ARG;
+}
+
+static int state_walk_any(const WalkArgs& a, int dtype, int mode, hipStream_t stream) {
+  if (a.n_entries <= 0) return SHARPI_OK;
+  if (a.nh <= 0 || a.nh > 65535 || a.n_entries > 65535 || a.dk <= 0 || a.dk > 256 || a.dv <= 0 || a.heads_per_group <= 0) return SHARPI_ERR_ARG;
+  if (mode != WALK_EXP_GATES && mode != WALK_STATE_SPACE) return SHARPI_ERR_ARG;
+  if (!a.gates || !a.p0 || !a.p1 || (mode == WALK_STATE_SPACE && !a.p2) || (mode == WALK_EXP_GATES && !(a.cap > 0.f))) return SHARPI_ERR_ARG;
+  if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;
+  if (a.segs && (!a.ent_segs || !a.seg_local || !a.seg_start || !a.seg_decay || a.n_segs < a.n_entries || a.n_segs > 65535)) return SHARPI_ERR_ARG;
+  if (mode == WALK_EXP_GATES) {
+    if (dtype == DT_F32) return launch_state_walk<float, WALK_EXP_GATES>(a, stream);
+    return launch_state_walk<bf16_t, WALK_EXP_GATES>(a, stream);
+  }
+  if (dtype == DT_F32) return launch_state_walk<float, WALK_STATE_SPACE>(a, stream);
+  return launch_state_walk<bf16_t, WALK_STATE_SPACE>(a, stream);
 }
 
 // proj [T, stride] (dtype): q and k of head h at columns q_off / k_off + (h / heads_per_group) dk, v at
@@ -234,21 +393,26 @@ SHARPI_EXPORT int sharpi_state_walk(const void* proj, int dtype, int stride, int
                                     const float* p1, const float* p2, float cap, float q_scale, int mode, float* state,
                                     const int* state_slots, const int* cu_tokens, float* out, int n_entries, int nh,
                                     int dk, int dv, hipStream_t stream) {
-  if (n_entries <= 0) return SHARPI_OK;
-  if (nh <= 0 || nh > 65535 || n_entries > 65535 || dk <= 0 || dk > 256 || dv <= 0 || heads_per_group <= 0) return SHARPI_ERR_ARG;
-  if (mode != WALK_EXP_GATES && mode != WALK_STATE_SPACE) return SHARPI_ERR_ARG;
-  if (!gates || !p0 || !p1 || (mode == WALK_STATE_SPACE && !p2) || (mode == WALK_EXP_GATES && !(cap > 0.f))) return SHARPI_ERR_ARG;
-  if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;
-#define GO(TT, MM)                                                                                                     \
-  return launch_state_walk<TT, MM>(proj, stride, q_off, k_off, v_off, heads_per_group, gates, gate_stride, p0, p1, p2, \
-                                   cap, q_scale, state, state_slots, cu_tokens, out, n_entries, nh, dk, dv, stream)
-  if (mode == WALK_EXP_GATES) {
-    if (dtype == DT_F32) GO(float, WALK_EXP_GATES);
-    GO(bf16_t, WALK_EXP_GATES);
-  }
-  if (dtype == DT_F32) GO(float, WALK_STATE_SPACE);
-  GO(bf16_t, WALK_STATE_SPACE);
-#undef GO
+  const WalkArgs a{proj, stride, q_off, k_off, v_off, heads_per_group, gates, gate_stride, p0, p1, p2, cap, q_scale, state,
+                   state_slots, cu_tokens, out, n_entries, nh, dk, dv, nullptr, nullptr, 0, nullptr, nullptr, nullptr};
+  return state_walk_any(a, dtype, mode, stream);
+}
+
+// The same walk with long entries cut into segments that are walked side by side (results equal to
+// rounding).  segs int [n_segs, 4] = (entry, first row, tokens, 1 if the entry's last), in the entries'
+// order; ent_segs int [n_entries, 2] = (first segment, segments); seg_local and seg_start float [n_segs, nh,
+// ceil(dv / 8), slice]; seg_decay float [n_segs, nh].
+SHARPI_EXPORT int sharpi_state_walk_segmented(const void* proj, int dtype, int stride, int q_off, int k_off, int v_off,
+                                              int heads_per_group, const float* gates, int gate_stride, const float* p0,
+                                              const float* p1, const float* p2, float cap, float q_scale, int mode,
+                                              float* state, const int* state_slots, const int* cu_tokens, float* out,
+                                              int n_entries, int nh, int dk, int dv, const int* segs, const int* ent_segs,
+                                              int n_segs, float* seg_local, float* seg_start, float* seg_decay,
+                                              hipStream_t stream) {
+  if (!segs) return SHARPI_ERR_ARG;
+  const WalkArgs a{proj, stride, q_off, k_off, v_off, heads_per_group, gates, gate_stride, p0, p1, p2, cap, q_scale, state,
+                   state_slots, cu_tokens, out, n_entries, nh, dk, dv, segs, ent_segs, n_segs, seg_local, seg_start, seg_decay};
+  return state_walk_any(a, dtype, mode, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -1551,7 +1551,8 @@ def walk_state_matrices(state: torch.Tensor, dk: int, dv: int, mode: int):
 
 
 def state_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, heads_per_group: int, gates: torch.Tensor,
-               params, cap: float, q_scale: float, mode: int, state: torch.Tensor, ctx, nh: int, dk: int, dv: int) -> torch.Tensor:
+               params, cap: float, q_scale: float, mode: int, state: torch.Tensor, ctx, nh: int, dk: int, dv: int,
+               segments=None) -> torch.Tensor:
     """The recurrence S_t = a_t S_(t-1) + b_t k_t v_t^T, o_t = S_t^T q_t per head with one decay a_t and one
     input weight b_t per (token, head), token by token along every entry of the step, from and into
     state [slots, *walk_state_shape(nh, dk, dv, mode)] (float32) at the entries' state slots.  q and k of
@@ -1565,7 +1566,11 @@ def state_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, heads_per
     * WALK_STATE_SPACE: gates column h is the step size before its softplus, params (its bias, A_log, D);
       a = exp(-exp(A_log) dt), b = dt, and the result is o + D v.
 
-    Returns float32 [T, nh * dv]."""
+    ``segments`` = (segs, ent_segs) on the device (see :func:`gla_segments`): long entries are then walked
+    segment by segment side by side.  A stretch of tokens acts on the state as S -> D S + L (D the product of
+    its decays, one number a head; L what it makes of a zero state), so every segment is first walked from
+    nothing, the true start states follow one from the other, and a second walk from those writes the
+    outputs (results equal to rounding).  Returns float32 [T, nh * dv]."""
     _dev(proj, gates, state, *params)
     T, N = proj.shape
     groups = nh // heads_per_group if heads_per_group > 0 else 0
@@ -1585,6 +1590,23 @@ def state_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, heads_per
           "state_walk: the step's per-entry arrays do not fit")
     out = torch.empty(T, nh * dv, dtype=torch.float32, device=proj.device)
     p = list(params) + [None] * (3 - n_par)
+    if segments is not None:
+        segs, ent_segs = segments
+        _dev(segs, ent_segs)
+        _i32(segs, "segs")
+        _i32(ent_segs, "ent_segs")
+        n_segs = segs.numel() // 4
+        _need(segs.numel() == 4 * n_segs and ent_segs.numel() == 2 * ctx.n_entries and n_segs >= ctx.n_entries,
+              "state_walk: segs [n, 4] and ent_segs [entries, 2] wanted")
+        shape = (n_segs,) + walk_state_shape(nh, dk, dv, mode)
+        seg_local = torch.empty(shape, dtype=torch.float32, device=proj.device)
+        seg_start = torch.empty(shape, dtype=torch.float32, device=proj.device)
+        seg_decay = torch.empty(n_segs, nh, dtype=torch.float32, device=proj.device)
+        _run("sharpi_state_walk_segmented", _ptr(proj), _code(proj.dtype), N, int(q_off), int(k_off), int(v_off),
+             int(heads_per_group), _ptr(gates), gates.shape[1], _ptr(p[0]), _ptr(p[1]), _ptr(p[2]), float(cap), float(q_scale),
+             int(mode), _ptr(state), _ptr(ctx.state_slots), _ptr(ctx.cu_tokens), _ptr(out), ctx.n_entries, nh, dk, dv,
+             _ptr(segs), _ptr(ent_segs), n_segs, _ptr(seg_local), _ptr(seg_start), _ptr(seg_decay), _stream())
+        return out
     _run("sharpi_state_walk", _ptr(proj), _code(proj.dtype), N, int(q_off), int(k_off), int(v_off), int(heads_per_group),
          _ptr(gates), gates.shape[1], _ptr(p[0]), _ptr(p[1]), _ptr(p[2]), float(cap), float(q_scale), int(mode), _ptr(state),
          _ptr(ctx.state_slots), _ptr(ctx.cu_tokens), _ptr(out), ctx.n_entries, nh, dk, dv, _stream())

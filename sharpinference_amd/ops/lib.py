@@ -59,6 +59,7 @@ _SIGNATURES = {
     "sharpi_norm_mean": [P, P, I, I, P, I, I, F, P],
     "sharpi_post_pre_norm": [P, P, P, I, I, P, P, P, I, I, I, F, P],
     "sharpi_state_walk": [P, I, I, I, I, I, I, P, I, P, P, P, F, F, I, P, P, P, P, I, I, I, I, P],
+    "sharpi_state_walk_segmented": [P, I, I, I, I, I, I, P, I, P, P, P, F, F, I, P, P, P, P, I, I, I, I, P, P, I, P, P, P, P],
     "sharpi_group_norm_gate": [P, P, F, P, I, I, I, I, I, P, I, I, I, P],
     "sharpi_short_conv": [P, I, I, I, P, P, I, P, P, P, P, P, I, I, I, I, P],
     "sharpi_sigmoid_gate": [P, P, I, I, I, P, I, I, P],

@@ -16,7 +16,7 @@ SEGMENT_UP_TO_BLOCKS = 2048   # ... and a layer walks in segments while whole en
 
 
 class WalkSegments(StepPlanner):
-    """The work lists of the segmented walk, made once a step for all linear-attention layers: none
+    """The work lists of the segmented walk, made once a step for all layers that walk a state: none
     unless some entry is long (decode steps and short portions are walked whole)."""
 
     key = "linear attention"
@@ -33,6 +33,7 @@ class WalkSegments(StepPlanner):
 
 
 _SEGMENTS = WalkSegments()
+WALK_SEGMENTS = _SEGMENTS         # every mixer that walks a state token by token shares the step's one list
 
 
 class GatedLinearAttention(Part):

@@ -10,6 +10,7 @@ from .. import ops
 from ..cache.spec import MixedSpec, StateSpec
 from ..ops.profile import section
 from .base import INIT_NORM_WEIGHT, LayerCache, ParamSpec, Part, StepContext, TensorSource
+from .linear_attention import SEGMENT_UP_TO_BLOCKS, WALK_SEGMENTS
 
 
 def _fuse(parts, hidden: int) -> torch.Tensor:
@@ -20,6 +21,13 @@ def _fuse(parts, hidden: int) -> torch.Tensor:
         fused[o:o + p.shape[0]].copy_(p)
         o += p.shape[0]
     return fused
+
+
+def _segments_for(ctx: StepContext, nh: int, dv: int):
+    """The step's segment lists where a walk of whole entries would leave the chip idle (a long entry alone
+    in its step), else None."""
+    whole_blocks = ctx.n_entries * nh * ((dv + ops.WALK_STATE_COLS - 1) // ops.WALK_STATE_COLS)
+    return ctx.extras.get(WALK_SEGMENTS.key) if whole_blocks < SEGMENT_UP_TO_BLOCKS else None
 
 
 class MatrixMemory(Part):
@@ -56,6 +64,9 @@ class MatrixMemory(Part):
         self.b_f: Optional[torch.Tensor] = None
         self.w_norm: Optional[torch.Tensor] = None    # float32 [heads * dv]
         self.w_o = None
+
+    def step_planners(self):
+        return (WALK_SEGMENTS,)
 
     def cache_spec(self) -> StateSpec:
         return StateSpec(ops.walk_state_shape(self.nh, self.dk, self.dv, ops.WALK_EXP_GATES), torch.float32)
@@ -100,7 +111,8 @@ class MatrixMemory(Part):
         with section("recurrence", nbytes=lambda: 8 * ctx.n_entries * qk * self.dv + T * (width * (2 * qk + vv) + 4 * vv),
                      flops=4.0 * T * qk * self.dv):
             o = ops.state_walk(proj, 0, qk, 2 * qk, 1, gates, (self.b_i, self.b_f), self.cap, self.dk ** -0.5,
-                               ops.WALK_EXP_GATES, state, ctx, self.nh, self.dk, self.dv)
+                               ops.WALK_EXP_GATES, state, ctx, self.nh, self.dk, self.dv,
+                               segments=_segments_for(ctx, self.nh, self.dv))
         with section("head norm + gate", nbytes=T * vv * (4 + 2 * width)):
             y = ops.group_norm_gate(o, self.w_norm, self.eps, self.nh, ctx.act_dtype, proj, 2 * qk + vv, ops.GATE_SIGMOID_ACT)
         with section("o", nbytes=width * self.hidden * (vv + T) + width * T * vv, flops=2.0 * T * self.hidden * vv):
@@ -146,6 +158,9 @@ class StateSpaceMixer(Part):
         self.d_skip: Optional[torch.Tensor] = None
         self.w_norm: Optional[torch.Tensor] = None
         self.w_o = None
+
+    def step_planners(self):
+        return (WALK_SEGMENTS,)
 
     def cache_spec(self):
         walk = StateSpec(ops.walk_state_shape(self.nh, self.N, self.dv, ops.WALK_STATE_SPACE), torch.float32)
@@ -200,7 +215,7 @@ class StateSpaceMixer(Part):
                      flops=4.0 * T * self.nh * self.N * self.dv):
             y = ops.state_walk(xbc, self.inner + self.G * self.N, self.inner, 0, self.nh // self.G, dt,
                                (self.dt_bias, self.a_log, self.d_skip), 0.0, 1.0, ops.WALK_STATE_SPACE, states[0], ctx,
-                               self.nh, self.N, self.dv)
+                               self.nh, self.N, self.dv, segments=_segments_for(ctx, self.nh, self.dv))
         with section("head norm + gate", nbytes=T * self.inner * (4 + 2 * width)):
             y = ops.group_norm_gate(y, self.w_norm, self.eps, self.norm_groups, ctx.act_dtype, proj, 0, ops.GATE_SILU, gate_first=True)
         with section("o", nbytes=width * self.hidden * (self.inner + T) + width * T * self.inner, flops=2.0 * T * self.hidden * self.inner):

@@ -267,6 +267,87 @@ def test_one_token_far_back_is_still_in_the_state(dtype, mode):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode, H, G, dk, dv", [("gates", 2, 2, 32, 16), ("gates", 3, 3, 72, 20), ("gates", 1, 1, 136, 9),
+                                               ("space", 4, 2, 48, 16), ("space", 2, 1, 128, 24), ("space", 3, 3, 10, 8)])
+def test_long_entries_walked_in_segments_side_by_side(dtype, mode, H, G, dk, dv):
+    """Three entries of 700, 5 and 257 tokens in one step, from states that earlier tokens left: cut into
+    segments (each walked from nothing, the start states made one from the other, then walked again)
+    against the plain recurrence over the whole sequences, and the states left in the slots against a
+    walk of whole entries."""
+    from sharpinference_amd import ops
+
+    g = torch.Generator().manual_seed(dk * dv)
+    before, lens, slots = [3, 40, 0], [700, 5, 257], [2, 0, 3]
+    state_mode = ops.WALK_EXP_GATES if mode == "gates" else ops.WALK_STATE_SPACE
+    cap = 6.0
+    n_gate = 2 * H if mode == "gates" else H
+    rows, zs = [], []
+    for b, n in zip(before, lens):
+        T = b + n
+        q, k, v = torch.randn(T, G * dk, generator=g) * 0.5, torch.randn(T, G * dk, generator=g) * 0.5, torch.randn(T, H * dv, generator=g)
+        rows.append((torch.cat([v, k, q], dim=1) if mode == "space" else torch.cat([q, k, v], dim=1)).to(DT[dtype]))
+        z = torch.randn(T, n_gate, generator=g) * 2.0
+        if mode == "gates":
+            z[:, H:] += 3.0                                       # forget gates mostly open: the far past still counts
+        else:
+            z -= 3.0                                              # small steps: slow decays
+        zs.append(z)
+    if mode == "gates":
+        par = (torch.randn(H, generator=g), torch.randn(H, generator=g))
+        offs, rep, scale = (0, G * dk, 2 * G * dk), 1, dk ** -0.5
+    else:
+        par = (torch.randn(H, generator=g) * 0.5, torch.randn(H, generator=g) * 0.5 - 1.0, torch.randn(H, generator=g))
+        offs, rep, scale = (H * dv + G * dk, H * dv, 0), H // G, 1.0
+    dpar = tuple(p.to(DEV) for p in par)
+
+    def run(segmented):
+        state = torch.zeros(4, *ops.walk_state_shape(H, dk, dv, state_mode), device=DEV)
+        outs = []
+        for part in (0, 1):                                       # what came before, then the long step
+            ns = [b if part == 0 else n for b, n in zip(before, lens)]
+            at = [0 if part == 0 else b for b in before]
+            live = [i for i, n in enumerate(ns) if n > 0]
+            ctx = _Step([ns[i] for i in live], [at[i] for i in live], [slots[i] for i in live])
+            x = torch.cat([rows[i][at[i]:at[i] + ns[i]] for i in live]).to(DEV)
+            z = torch.cat([zs[i][at[i]:at[i] + ns[i]] for i in live]).to(DEV)
+            segments = None
+            if segmented and part == 1:
+                segs, ents = ops.gla_segments(ctx_lens := [ns[i] for i in live], ctx.cu_tokens.cpu().numpy())
+                assert segs.shape[0] == sum((n + 127) // 128 for n in ctx_lens)
+                segments = (torch.from_numpy(segs).to(DEV), torch.from_numpy(ents).to(DEV))
+            o = ops.state_walk(x, offs[0], offs[1], offs[2], rep, z, dpar, cap, scale, state_mode, state, ctx, H, dk, dv,
+                               segments=segments)
+            outs.append((live, [ns[i] for i in live], o.cpu()))
+        return outs[1], state
+
+    (live, ns, seg_out), seg_state = run(True)
+    (_, _, whole_out), whole_state = run(False)
+    o = 0
+    for i, n in zip(live, ns):
+        p, z = rows[i].double(), zs[i].double()
+        T = p.shape[0]
+        if mode == "gates":
+            log_i = P.capped(z[:, :H] + par[0].double(), cap)
+            log_f = P.log_sigmoid(P.capped(z[:, H:] + par[1].double(), cap))
+            want = P.matrix_memory(p[:, :H * dk].reshape(T, H, dk) * scale, p[:, H * dk:2 * H * dk].reshape(T, H, dk),
+                                   p[:, 2 * H * dk:].reshape(T, H, dv), log_i, log_f)
+        else:
+            want = P.state_space_scan(p[:, :H * dv].reshape(T, H, dv), p[:, H * dv:H * dv + G * dk].reshape(T, G, dk),
+                                      p[:, H * dv + G * dk:].reshape(T, G, dk), P.softplus(z + par[0].double()), par[1].double(),
+                                      par[2].double())
+        want = want.reshape(T, -1)[before[i]:]
+        assert _rel_rms(seg_out[o:o + n], want) < FLOAT_LONG_WALK, f"entry {i}"
+        assert _rel_rms(whole_out[o:o + n], want) < FLOAT_LONG_WALK, f"entry {i} whole"
+        o += n
+    for slot in slots:
+        for a, b in zip(ops.walk_state_matrices(seg_state[slot], dk, dv, state_mode), ops.walk_state_matrices(whole_state[slot], dk, dv, state_mode)):
+            if a is not None:
+                scale_of = float(b.abs().max()) + 1e-30
+                assert float((a - b).abs().max()) / scale_of < FLOAT_WALK, f"slot {slot}"
+    assert float(seg_state[1].abs().max()) == 0.0                 # the slot no entry names
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("channels, taps, bias", [(29, 2, True), (64, 3, True), (200, 4, True), (24, 8, True), (40, 1, True), (16, 4, False)])
 def test_the_biased_convolution_carries_its_tail_from_step_to_step(dtype, channels, taps, bias):
     """Three requests over five steps, portions shorter than the convolution's reach among them:

@@ -40,7 +40,7 @@ def _both(lib, c):
     """(existing entry point's output, the new one's) for one case."""
     P, I, F = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
     old = lib.sharpi_attention_decode
-    old.argtypes = [P] * 10 + [I, I, F] + [I] * 8 + [F, I, P]      # (..., softcap, sink, stream)
+    old.argtypes = [P] * 10 + [I, I, F] + [I] * 8 + [F, I, P, P]   # (..., softcap, sink, sink_vals, stream)
     old.restype = I
     new = lib.sharpi_attention_decode_noalloc
     new.argtypes = [P] * 8 + [I, I, F] + [I] * 8 + [P]
@@ -53,7 +53,7 @@ def _both(lib, c):
     tail = (c["wk"], c["w"], c["scale"], c["n"], c["nh"], c["nkv"], c["hd"], c["ps"], c["maxb"], c["pages"], c["splits"], stream)
     head = (c["q"].data_ptr(), c["k"].data_ptr(), c["v"].data_ptr(), c["table"].data_ptr(), c["ent"].data_ptr(),
             c["pos"].data_ptr(), None)
-    rc = old(*head, part_o.data_ptr(), part_ml.data_ptr(), out_old.data_ptr(), *tail[:-1], 0.0, 0, stream)
+    rc = old(*head, part_o.data_ptr(), part_ml.data_ptr(), out_old.data_ptr(), *tail[:-1], 0.0, 0, None, stream)
     assert rc == 0, rc
     rc = new(*head, out_new.data_ptr(), *tail)
     assert rc == 0, rc
