@@ -17,11 +17,39 @@ __global__ __launch_bounds__(256) void sigmoid_gate_kernel(const T* __restrict__
   }
 }
 
+// eight elements a thread, 16-byte accesses (N, stride and g_off multiples of 8)
+template <typename T>
+__global__ __launch_bounds__(256) void sigmoid_gate8_kernel(const T* __restrict__ x, const T* __restrict__ proj, int stride,
+                                                             int g_off, T* __restrict__ out, int n_tokens, int N) {
+  const int per_row = N >> 3;
+  const size_t total = (size_t)n_tokens * per_row;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = i / per_row, c = (i % per_row) << 3;
+    float z[8], v[8];
+    load8(proj + t * stride + g_off + c, z);
+    load8(x + t * N + c, v);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = v[k] / (1.0f + expf(-z[k]));
+    store8(out + t * N + c, v);
+  }
+}
+
 SHARPI_EXPORT int sharpi_sigmoid_gate(const void* x, const void* proj, int dtype, int stride, int g_off, void* out,
                                       int n_tokens, int N, hipStream_t stream) {
   if (n_tokens <= 0) return SHARPI_OK;
   if (N <= 0 || g_off < 0 || g_off + N > stride) return SHARPI_ERR_ARG;
   const size_t total = (size_t)n_tokens * N;
+  const bool by8 = N % 8 == 0 && stride % 8 == 0 && g_off % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 32 == 0 &&
+                   reinterpret_cast<uintptr_t>(proj) % 32 == 0 && reinterpret_cast<uintptr_t>(out) % 32 == 0;
+  if (by8 && (dtype == DT_F32 || dtype == DT_BF16)) {
+    const dim3 block8(256), grid8((unsigned)min((size_t)16384, (total / 8 + 255) / 256));
+    if (dtype == DT_F32)
+      sigmoid_gate8_kernel<float><<<grid8, block8, 0, stream>>>((const float*)x, (const float*)proj, stride, g_off, (float*)out, n_tokens, N);
+    else
+      sigmoid_gate8_kernel<bf16_t><<<grid8, block8, 0, stream>>>((const bf16_t*)x, (const bf16_t*)proj, stride, g_off, (bf16_t*)out, n_tokens, N);
+    SHARPI_CHECK_LAUNCH();
+    return SHARPI_OK;
+  }
   const dim3 block(256), grid((unsigned)min((size_t)8192, (total + 255) / 256));
   if (dtype == DT_F32)
     sigmoid_gate_kernel<float><<<grid, block, 0, stream>>>((const float*)x, (const float*)proj, stride, g_off, (float*)out, n_tokens, N);

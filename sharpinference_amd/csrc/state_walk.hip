@@ -280,44 +280,60 @@ __global__ __launch_bounds__(kWave) void state_walk_kernel(
 }
 
 // The segments' start states, one entry's after the other: start(first) = the slot's state, start(s + 1) =
-// what segment s makes of start(s).  A block = (8 value columns, head, entry); a lane moves the floats
-// lane, lane + 64, .. of the slice (S and, for the gates, n; each lane reads only what it wrote).
+// what segment s makes of start(s).  A thread owns one float of a (head, 8 value columns) slice (of S or,
+// for the gates, of n) and keeps it in a register; it asks for eight segments' local values before it
+// uses the first (they do not depend on the chain), then moves along them.
+constexpr int kCombineThreads = 256;
+constexpr int kCombineAhead = 8;
+
 template <int MODE>
-__global__ __launch_bounds__(kWave) void state_walk_combine_kernel(
+__global__ __launch_bounds__(kCombineThreads) void state_walk_combine_kernel(
     const float* __restrict__ state, const int* __restrict__ state_slots, const int* __restrict__ ent_segs,
     const float* __restrict__ seg_local, float* __restrict__ seg_start, const float* __restrict__ seg_decay, int nh,
     int ncb, int dkp) {
-  const int cb = blockIdx.x, h = blockIdx.y, e = blockIdx.z, lane = threadIdx.x;
+  const int h = blockIdx.y, e = blockIdx.z;
   const int first = ent_segs[2 * e], count = ent_segs[2 * e + 1];
   if (count <= 0) return;
   const int slice = walk_slice_floats(dkp, MODE);
-  const int moved = (dkp / 8) * 64 + (MODE == WALK_EXP_GATES ? dkp : 0);     // S and n
-  const float* slot = state + (((size_t)state_slots[e] * nh + h) * ncb + cb) * slice;
-  float* cur = seg_start + (((size_t)first * nh + h) * ncb + cb) * slice;
-  for (int i = lane; i < moved; i += kWave) cur[i] = slot[i];
-  float m = 0.f;
-  if (MODE == WALK_EXP_GATES) {
-    m = slot[moved];
-    if (lane == 0) cur[moved] = m;
-  }
-  for (int s = first; s + 1 < first + count; ++s) {
-    const size_t at = (((size_t)s * nh + h) * ncb + cb) * slice;
-    const float* loc = seg_local + at;
-    float* next = seg_start + at + (size_t)nh * ncb * slice;
-    const float F = seg_decay[(size_t)s * nh + h];
-    float wa, wb = 1.f;
-    if (MODE == WALK_EXP_GATES) {
-      const float m_loc = loc[moved];
-      const float m_new = fmaxf(F + m, m_loc);
-      wa = expf(F + m - m_new);
-      wb = expf(m_loc - m_new);
-      m = m_new;
-      if (lane == 0) next[moved] = m;
-    } else {
-      wa = expf(F);
+  const int moved = (dkp / 8) * 64 + (MODE == WALK_EXP_GATES ? dkp : 0);     // S and n; the maximum lies behind them
+  const int idx = blockIdx.x * kCombineThreads + threadIdx.x;              // over the head's slices
+  if (idx >= ncb * moved) return;
+  const int cb = idx / moved, i = idx % moved;
+  const size_t per_seg = (size_t)nh * ncb * slice;
+  const size_t at = ((size_t)h * ncb + cb) * slice;
+  const float* slot = state + (size_t)state_slots[e] * per_seg + at;
+  float cur = slot[i];
+  float m = MODE == WALK_EXP_GATES ? slot[moved] : 0.f;
+  seg_start[(size_t)first * per_seg + at + i] = cur;
+  if (MODE == WALK_EXP_GATES && i == 0) seg_start[(size_t)first * per_seg + at + moved] = m;
+  for (int s0 = first; s0 + 1 < first + count; s0 += kCombineAhead) {
+    const int n = min(kCombineAhead, first + count - 1 - s0);
+    float loc[kCombineAhead], F[kCombineAhead], m_loc[kCombineAhead];
+#pragma unroll
+    for (int u = 0; u < kCombineAhead; ++u) {
+      const int s = s0 + min(u, n - 1);                // (addresses clamped: no load behind a branch)
+      loc[u] = seg_local[(size_t)s * per_seg + at + i];
+      F[u] = seg_decay[(size_t)s * nh + h];
+      m_loc[u] = MODE == WALK_EXP_GATES ? seg_local[(size_t)s * per_seg + at + moved] : 0.f;
     }
-    for (int i = lane; i < moved; i += kWave) next[i] = fmaf(wa, cur[i], wb * loc[i]);
-    cur = next;
+#pragma unroll
+    for (int u = 0; u < kCombineAhead; ++u) {
+      if (u < n) {
+        float wa, wb = 1.f;
+        if (MODE == WALK_EXP_GATES) {
+          const float m_new = fmaxf(F[u] + m, m_loc[u]);
+          wa = expf(F[u] + m - m_new);
+          wb = expf(m_loc[u] - m_new);
+          m = m_new;
+        } else {
+          wa = expf(F[u]);
+        }
+        cur = fmaf(wa, cur, wb * loc[u]);
+        const size_t to = (size_t)(s0 + u + 1) * per_seg + at;
+        seg_start[to + i] = cur;
+        if (MODE == WALK_EXP_GATES && i == 0) seg_start[to + moved] = m;
+      }
+    }
   }
 }
 
@@ -347,7 +363,8 @@ static int launch_walk_rpl(const WalkArgs& a, int ncb, int vec, hipStream_t stre
   }
   launch_walk_phase<T, RPL, MODE, WALK_LOCAL>(a, ncb, vec, stream);
   SHARPI_CHECK_LAUNCH();
-  state_walk_combine_kernel<MODE><<<dim3(ncb, a.nh, a.n_entries), kWave, 0, stream>>>(
+  const int moved = RPL * 64 + (MODE == WALK_EXP_GATES ? RPL * 8 : 0);
+  state_walk_combine_kernel<MODE><<<dim3(ceil_div(ncb * moved, kCombineThreads), a.nh, a.n_entries), kCombineThreads, 0, stream>>>(
       a.state, a.state_slots, a.ent_segs, a.seg_local, a.seg_start, a.seg_decay, a.nh, ncb, RPL * 8);
   SHARPI_CHECK_LAUNCH();
   launch_walk_phase<T, RPL, MODE, WALK_FINAL>(a, ncb, vec, stream);
