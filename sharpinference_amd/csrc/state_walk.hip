@@ -15,9 +15,11 @@
 //
 // Work: a block (one wave) = (entry, head, 8 value columns).  Lane (g, j) keeps RPL = DKP / 8 rows
 // g RPL .. g RPL + RPL - 1 of column j in registers (DKP = dk rounded up to 32, 64, 128 or 256; rows
-// beyond dk stay zero).  Tokens are staged 16 at a time into LDS: q and k as floats in the order the
-// lanes read them, the 16 tokens' gates computed side by side (the running maximum by a scan over
-// the lanes whose order is fixed by the chunk), then the wave walks the 16 tokens.  A request's
+// beyond dk stay zero).  Tokens are staged 8 at a time into LDS (8 KB a block at 128 rows: with 16 a
+// CU held ten waves and the walk took 1.4 times as long; with 4 the gates' arithmetic, done once a
+// stage, weighs more): q and k as floats in the order the
+// lanes read them, the stage's gates computed side by side (the running maximum by a scan over
+// the lanes whose order is fixed by the chunk), then the wave walks the stage's tokens.  A request's
 // state lies slice by slice, [heads, ceil(dv / 8), slice], a slice = RPL x 64 floats of S in the
 // lanes' order (row g RPL + r of column j at r 64 + 8 g + j), and, for the exponential gates, DKP
 // floats of n and the maximum m (each slice its own copy: the blocks of a head do not wait for
@@ -37,7 +39,7 @@
 enum : int { WALK_EXP_GATES = 0, WALK_STATE_SPACE = 1 };
 enum : int { WALK_WHOLE = 0, WALK_LOCAL = 1, WALK_FINAL = 2 };
 constexpr int kWalkCols = 8;       // value columns of a block
-constexpr int kWalkChunk = 16;     // tokens staged at a time
+constexpr int kWalkChunk = 8;      // tokens staged at a time
 constexpr float kWalkFloor = 1e-6f;
 
 SHARPI_EXPORT int sharpi_state_walk_cols() { return kWalkCols; }
@@ -79,7 +81,7 @@ __global__ __launch_bounds__(kWave) void state_walk_kernel(
     const float* __restrict__ seg_start, float* __restrict__ seg_decay) {
   constexpr int DKP = RPL * 8;
   constexpr int V = 16 / (int)sizeof(T);            // elements of a 16-byte load
-  __shared__ __attribute__((aligned(16))) float q_s[kWalkChunk][DKP];
+  __shared__ __attribute__((aligned(16))) float q_s[PHASE == WALK_LOCAL ? 1 : kWalkChunk][DKP];     // (no outputs, no queries)
   __shared__ __attribute__((aligned(16))) float k_s[kWalkChunk][DKP];
   __shared__ float v_s[kWalkChunk][kWalkCols];
   __shared__ float a_s[kWalkChunk], b_s[kWalkChunk], e_s[kWalkChunk];
@@ -155,7 +157,7 @@ __global__ __launch_bounds__(kWave) void state_walk_kernel(
 #pragma unroll
         for (int i = 0; i < V; i += 4) {             // four rows of a lane lie together
           const int at = staged_at<RPL>(row0 + i);
-          *reinterpret_cast<float4*>(&q_s[tt][at]) = make_float4(qv[i] * q_scale, qv[i + 1] * q_scale, qv[i + 2] * q_scale, qv[i + 3] * q_scale);
+          if (PHASE != WALK_LOCAL) *reinterpret_cast<float4*>(&q_s[tt][at]) = make_float4(qv[i] * q_scale, qv[i + 1] * q_scale, qv[i + 2] * q_scale, qv[i + 3] * q_scale);
           *reinterpret_cast<float4*>(&k_s[tt][at]) = make_float4(kv[i], kv[i + 1], kv[i + 2], kv[i + 3]);
         }
       }
@@ -169,7 +171,7 @@ __global__ __launch_bounds__(kWave) void state_walk_kernel(
         kv = to_f32<T>(base[k_off]);
       }
       const int at = staged_at<RPL>(row);
-      q_s[tt][at] = qv;
+      if (PHASE != WALK_LOCAL) q_s[tt][at] = qv;
       k_s[tt][at] = kv;
     }
     for (int idx = lane; idx < kWalkChunk * kWalkCols; idx += kWave) {
@@ -230,7 +232,7 @@ __global__ __launch_bounds__(kWave) void state_walk_kernel(
       const float bv = b * vj;
       float acc = 0.f, nq = 0.f;
       const float4* k4 = reinterpret_cast<const float4*>(&k_s[tt][0]);
-      const float4* q4 = reinterpret_cast<const float4*>(&q_s[tt][0]);
+      const float4* q4 = reinterpret_cast<const float4*>(&q_s[PHASE == WALK_LOCAL ? 0 : tt][0]);
 #pragma unroll
       for (int r4 = 0; r4 < RPL / 4; ++r4) {
         const float4 kk = k4[r4 * 8 + g], qq = q4[r4 * 8 + g];
