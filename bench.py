@@ -626,14 +626,14 @@ NOSEDRA_KINDS = ["parallel", "parallel", "mamba2", "parallel"]
 
 def nosedra_config(z: dict) -> dict:
     left = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
-            "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 2.0}}}
-    right = {"heads": z["heads"], "dim": 128, "vdim": 128, "gate_cap": 15.0}
+            "rot": {"base": 1000000.0, "dims": 64, "scaling": {"factor": 4.0}}}
+    right = {"heads": z["heads"], "dim": 128, "vdim": 128, "gate_cap": 10.0}
     space = {"heads": 2 * z["width"] // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}
     mlp = {"kind": "dense", "ff": z["ff"]}
     layers = [{"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}, "mlp": mlp}
               if kind == "parallel" else {"type": "mamba2", "mixer": space, "mlp": mlp} for kind in NOSEDRA_KINDS[:z["layers"]]]
     return {"architecture": "Nosedra", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-5},
-            "token_side": {"dim": z["side"]}, "logit_softcap": 30.0, "layers": layers}
+            "token_side": {"dim": z["side"]}, "logit_softcap": 50.0, "layers": layers}
 
 
 def pazatar_like_nosedra(z: dict) -> dict:

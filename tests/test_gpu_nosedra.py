@@ -98,7 +98,7 @@ def _walk_plan(rows_of, gates_of, call):
 # the mechanisms alone
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("H, dk, dv, cap", [(2, 10, 24, 6.0), (6, 32, 48, 15.0), (1, 136, 20, 4.0), (3, 72, 50, 1.0), (2, 256, 16, 30.0),
+@pytest.mark.parametrize("H, dk, dv, cap", [(2, 10, 24, 6.0), (5, 32, 40, 12.0), (1, 136, 20, 4.0), (3, 72, 50, 1.0), (2, 256, 16, 30.0),
                                             (4, 64, 33, 8.0)])
 def test_the_matrix_memory_walks_every_entry_from_its_slots_state(dtype, H, dk, dv, cap):
     """Exponential gates with their cap, the running maximum from 0, the normaliser and the floor of
@@ -180,7 +180,7 @@ def test_the_matrix_memorys_first_tokens_and_its_denominators_floor(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("H, G, N, dv", [(3, 1, 10, 8), (4, 2, 48, 32), (8, 2, 64, 16), (2, 1, 72, 50), (3, 3, 136, 12), (4, 4, 20, 6),
+@pytest.mark.parametrize("H, G, N, dv", [(3, 1, 10, 8), (6, 2, 40, 24), (8, 2, 64, 16), (2, 1, 72, 50), (3, 3, 136, 12), (4, 4, 20, 6),
                                          (2, 2, 256, 9)])
 def test_the_state_space_walks_every_entry_from_its_slots_state(dtype, H, G, N, dv):
     """Step sizes through their softplus (no clamp: some far below 0, some large), decays
@@ -242,11 +242,11 @@ def test_one_token_far_back_is_still_in_the_state(dtype, mode):
         proj = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], dim=1).to(DT[dtype])
         zero = torch.zeros(H, device=DEV)
         for a, b in zip(cuts, cuts[1:]):
-            outs.append(ops.state_walk(proj[a:b].to(DEV), 0, H * dk, 2 * H * dk, 1, z[a:b].to(DEV), (zero, zero), 15.0, 1.0,
+            outs.append(ops.state_walk(proj[a:b].to(DEV), 0, H * dk, 2 * H * dk, 1, z[a:b].to(DEV), (zero, zero), 14.0, 1.0,
                                        state_mode, state, ctx_of(a, b), H, dk, dv).cpu())
         p = proj.double()
         want = P.matrix_memory(p[:, :H * dk].reshape(T, H, dk), p[:, H * dk:2 * H * dk].reshape(T, H, dk), p[:, 2 * H * dk:].reshape(T, H, dv),
-                               P.capped(z[:, :H].double(), 15.0), P.log_sigmoid(P.capped(z[:, H:].double(), 15.0)))
+                               P.capped(z[:, :H].double(), 14.0), P.log_sigmoid(P.capped(z[:, H:].double(), 14.0)))
     else:
         z = torch.full((T, H), -9.0)                              # dt = softplus(-9): tiny steps, decays almost 1
         z[mark] = 1.0
@@ -268,7 +268,7 @@ def test_one_token_far_back_is_still_in_the_state(dtype, mode):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("mode, H, G, dk, dv", [("gates", 2, 2, 32, 16), ("gates", 3, 3, 72, 20), ("gates", 1, 1, 136, 9),
-                                               ("space", 4, 2, 48, 16), ("space", 2, 1, 128, 24), ("space", 3, 3, 10, 8)])
+                                               ("space", 4, 2, 40, 16), ("space", 2, 1, 128, 24), ("space", 3, 3, 10, 8)])
 def test_long_entries_walked_in_segments_side_by_side(dtype, mode, H, G, dk, dv):
     """Three entries of 700, 5 and 257 tokens in one step, from states that earlier tokens left: cut into
     segments (each walked from nothing, the start states made one from the other, then walked again)
@@ -381,7 +381,7 @@ def test_the_biased_convolution_carries_its_tail_from_step_to_step(dtype, channe
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("T, groups, size, act, first", [(1, 6, 48, "sigmoid", False), (19, 2, 64, "silu", True), (70, 3, 8, "silu", True),
+@pytest.mark.parametrize("T, groups, size, act, first", [(1, 5, 40, "sigmoid", False), (19, 2, 64, "silu", True), (70, 3, 8, "silu", True),
                                                          (9, 1, 100, "silu", True), (33, 2, 50, "sigmoid", False), (5, 4, 6, "silu", False)])
 def test_parts_normed_each_by_its_own_rms_with_a_gate_before_or_after(dtype, T, groups, size, act, first):
     from sharpinference_amd import ops
@@ -417,8 +417,8 @@ def test_a_scaled_sum_of_branches_joins_the_stream_in_float(dtype, T, N):
     h = torch.randn(T, N, generator=g) * 3
     a, b = torch.randn(T, N, generator=g).to(DT[dtype]), torch.randn(T, N, generator=g).to(DT[dtype])
     hd = h.clone().to(DEV)
-    out = ops.stream_add(hd, ops.BranchSum([a.to(DEV), b.to(DEV)], (1.2, -0.7)), DT[dtype])
-    want = h.double() + 1.2 * a.double() + -0.7 * b.double()
+    out = ops.stream_add(hd, ops.BranchSum([a.to(DEV), b.to(DEV)], (1.3, -0.7)), DT[dtype])
+    want = h.double() + 1.3 * a.double() + -0.7 * b.double()
     assert _rel_rms(hd, want) < 2e-6                             # the stream itself stays float
     assert out.dtype == DT[dtype] and _rel_rms(out, want) < (2e-6 if dtype == "float32" else 5e-3)
     alone = ops.BranchSum([a.to(DEV), b.to(DEV)], (0.5, 2.0)).tensor()
@@ -460,7 +460,7 @@ def test_the_token_input_the_biased_feed_forward_and_the_output_gate(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("H, G, d, e, dims, factor", [(4, 2, 12, 20, 4, 4.0), (6, 1, 8, 6, 8, 1.0), (8, 1, 128, 128, 64, 2.0), (4, 2, 64, 64, 64, 8.0),
+@pytest.mark.parametrize("H, G, d, e, dims, factor", [(4, 2, 12, 20, 4, 4.0), (6, 1, 8, 6, 8, 1.0), (8, 2, 128, 128, 32, 4.0), (4, 2, 64, 64, 64, 8.0),
                                                       (2, 1, 24, 40, 24, 1.5), (4, 4, 16, 16, 0, 1.0), (8, 2, 32, 32, 16, 2.0)])
 def test_split_half_rotation_then_unit_norm_and_the_cache_write(dtype, H, G, d, e, dims, factor):
     """Two requests in two steps each on shuffled pages: rotated (leading `dims` elements, halves
@@ -587,7 +587,7 @@ def _attend(q, kc, vc, bt, positions, how, scale, H, G, d, e, sink):
 
 
 @pytest.mark.parametrize("dtype, kernel, how", KERNELS)
-@pytest.mark.parametrize("S, H, G, d, e", [(70, 4, 2, 64, 64), (200, 8, 1, 128, 128), (131, 2, 1, 32, 32), (90, 6, 6, 64, 64), (50, 4, 2, 12, 20),
+@pytest.mark.parametrize("S, H, G, d, e", [(70, 4, 2, 64, 64), (200, 8, 2, 128, 128), (131, 2, 1, 32, 32), (90, 6, 6, 64, 64), (50, 4, 2, 12, 20),
                                            (77, 6, 1, 8, 6)])
 def test_attention_with_a_learned_sink_per_head(dtype, kernel, how, S, H, G, d, e):
     """Sinks from far below the scores (no effect) to far above (the head's output shrinks to

@@ -47,7 +47,7 @@ ODD = {
 EVEN = {
     "architecture": "Nosedra", "vocab": 256, "width": 128, "norm": {"eps": 1e-6}, "token_side": {"dim": 16},
     "layers": [
-        _parallel(_left(4, 2, 64, 64, 0.125, rot=(20000.0, 64, 8.0)), _right(4, 32, 32, 15.0), 1.2, 0.9, 256),
+        _parallel(_left(4, 2, 64, 64, 0.125, rot=(20000.0, 64, 8.0)), _right(4, 32, 32, 12.0), 1.1, 0.8, 256),
         _ssm(8, 16, 64, 2, 4, 4, 128),
         _parallel(_left(8, 2, 32, 32, 0.18, rot=(10000.0, 16, 2.0)), _right(2, 64, 64, 8.0), 1.0, 1.0, 64),
     ],
