@@ -78,12 +78,30 @@ __device__ __forceinline__ void store8(bf16_t* p, const float* v) {
 // the caller passes (shared with the Python side): SiLU x / (1 + exp(-x)), or GELU in its tanh form
 // 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))).  One definition for the activation kernel and
 // for the products that apply it in their epilogue, so both give the same bits.
-enum : int { ACT_SILU = 1, ACT_GELU_TANH = 2 };
-static inline __host__ __device__ bool act_known(int act) { return act == ACT_SILU || act == ACT_GELU_TANH; }
-__device__ __forceinline__ float gated_f32(int act, float g, float u, float s, bool scaled) {
+// ACT_SWISH_CLAMP is the clamped form: g = min(g, limit), u = clamp(u, -limit, limit), then
+// g sigmoid(1.702 g) * (u + 1); its limit travels beside the code (GatedAct).
+enum : int { ACT_SILU = 1, ACT_GELU_TANH = 2, ACT_SWISH_CLAMP = 3 };
+constexpr float kSwishSlope = 1.702f;
+struct GatedAct {
+  int code;
+  float limit;      // ACT_SWISH_CLAMP only
+};
+static inline __host__ __device__ bool act_known(int act) {
+  return act == ACT_SILU || act == ACT_GELU_TANH || act == ACT_SWISH_CLAMP;
+}
+static inline __host__ __device__ bool act_known(GatedAct a) {
+  return act_known(a.code) && (a.code != ACT_SWISH_CLAMP || a.limit > 0.f);
+}
+__device__ __forceinline__ float gated_f32(GatedAct actp, float g, float u, float s, bool scaled) {
+  const int act = actp.code;
   if (scaled) {
     g *= s;
     u *= s;
+  }
+  if (act == ACT_SWISH_CLAMP) {
+    g = fminf(g, actp.limit);
+    u = fminf(fmaxf(u, -actp.limit), actp.limit);
+    return (g / (1.0f + expf(-kSwishSlope * g))) * (u + 1.0f);
   }
   if (act == ACT_GELU_TANH) {
     const float t = tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g));

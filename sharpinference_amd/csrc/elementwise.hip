@@ -267,7 +267,7 @@ SHARPI_EXPORT int sharpi_add_rmsnorm(float* h, const void* delta, int delta_dtyp
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void silu_mul_kernel(const T* __restrict__ gu, const float* __restrict__ scale,
-                                T* __restrict__ out, int inter, int act, const float* __restrict__ bias) {
+                                T* __restrict__ out, int inter, GatedAct act, const float* __restrict__ bias) {
   const int m = blockIdx.x;
   const int i = blockIdx.y * blockDim.x + threadIdx.x;
   if (i >= inter) return;
@@ -283,7 +283,7 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, const float* __restric
 
 template <typename T>
 __global__ void silu_mul_vec_kernel(const T* __restrict__ gu, const float* __restrict__ scale,
-                                    T* __restrict__ out, int inter, int act, const float* __restrict__ bias) {
+                                    T* __restrict__ out, int inter, GatedAct act, const float* __restrict__ bias) {
   const int m = blockIdx.x;
   const int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
   if (i >= inter) return;
@@ -305,8 +305,9 @@ __global__ void silu_mul_vec_kernel(const T* __restrict__ gu, const float* __res
 }
 
 SHARPI_EXPORT int sharpi_silu_mul(const void* gu, const float* scale, void* out, int dtype, int rows, int inter,
-                                  int act, const float* bias, hipStream_t stream) {
+                                  int act_code, float act_limit, const float* bias, hipStream_t stream) {
   if (rows <= 0) return SHARPI_OK;
+  const GatedAct act{act_code, act_limit};
   if (inter <= 0 || ceil_div(inter, 256) > 65535 || !act_known(act)) return SHARPI_ERR_ARG;
   dim3 block(256), grid(rows, ceil_div(inter, 256));
   if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;

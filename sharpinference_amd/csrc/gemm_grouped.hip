@@ -17,7 +17,7 @@ SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, int x_rows, const void* W, 
   const dim3 grid = grouped_grid(n_rows, n_groups, nb, max_blocks), block(GW * kWave);
 #define GG_LAUNCH(TOV, PK)                                                                                             \
   grouped_gemm_kernel<TOV, kMaxNT, PK, false><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W, (TOV*)out, \
-                                                                         N, K, a_rows, nullptr, 0, group_offsets, plan, \
+                                                                         N, K, a_rows, nullptr, GatedAct{0, 0.f}, group_offsets, plan, \
                                                                          n_groups, nb)
   if (out_dtype == DT_BF16) {
     if (packed) GG_LAUNCH(bf16_t, true); else GG_LAUNCH(bf16_t, false);

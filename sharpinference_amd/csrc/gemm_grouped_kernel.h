@@ -96,7 +96,7 @@ template <bool STREAM> __device__ __forceinline__ bf16x8 load_weights(const bf16
 template <typename TO, int MT, int NT, bool PACKED, bool ACT, bool STREAM>
 __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const bf16_t* __restrict__ We,
                                              TO* __restrict__ out, int N, int K, const int* __restrict__ a_rows,
-                                             const float* __restrict__ act_scale, int act, int row0, int row_end,
+                                             const float* __restrict__ act_scale, GatedAct act, int row0, int row_end,
                                              int n_base, bf16_t (*xs)[GM][GPAD]) {
   static_assert(!ACT || NT % 2 == 0, "the SwiGLU form pairs gate tiles with up tiles");
   constexpr int HT = ACT ? NT / 2 : NT;         // tiles of distinct output columns per wave
@@ -279,7 +279,7 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
 template <typename TO, int NT, bool PACKED, bool ACT>
 __global__ __launch_bounds__(GW* kWave, 2) void grouped_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int N, int K,
-    const int* __restrict__ a_rows, const float* __restrict__ act_scale, int act,
+    const int* __restrict__ a_rows, const float* __restrict__ act_scale, GatedAct act,
     const int* __restrict__ group_offsets, const int* __restrict__ plan, int n_groups, int nb) {
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][GM][GPAD];
   __shared__ int s_slot;

@@ -8,9 +8,10 @@
 // (common.h).  N % 32 == 0; the rest as above.
 SHARPI_EXPORT int sharpi_gemm_grouped_swiglu(const void* x, int x_rows, const void* W, void* out, int n_rows, int N,
                                              int K, const int* a_rows, const int* group_offsets, const int* plan,
-                                             int n_groups, const float* act_scale, int packed, int act,
-                                             int max_blocks, hipStream_t stream) {
+                                             int n_groups, const float* act_scale, int packed, int act_code,
+                                             float act_limit, int max_blocks, hipStream_t stream) {
   if (n_rows <= 0) return SHARPI_OK;
+  const GatedAct act{act_code, act_limit};
   if (!act_known(act)) return SHARPI_ERR_ARG;
   if ((N & 31) || !grouped_args_ok(x_rows, n_rows, N, K, n_groups, packed, group_offsets, plan)) return SHARPI_ERR_ARG;
   constexpr int GN = columns_of(kMaxNT);   // the gated form pairs gate tiles with up tiles

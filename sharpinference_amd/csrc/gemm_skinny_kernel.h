@@ -72,7 +72,7 @@ template <int R, int MB, int NW, typename TO, bool ACT, bool PACKED>
 __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int M, int N, int K,
     const int* __restrict__ a_rows, const int* __restrict__ group_offsets, const float* __restrict__ act_scale,
-    int act, Picks pk) {
+    GatedAct act, Picks pk) {
   static_assert(!ACT || R % 2 == 0, "the SwiGLU form pairs gate and up tiles");
   constexpr int RT = ACT ? R : kRedTiles;   // tiles that meet in LDS per round
   constexpr int TG = ACT ? R / 2 : R;       // tiles of distinct output columns per block
@@ -321,7 +321,7 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
 template <int R, int MB, int NW, bool ACT, bool PACKED>
 static inline int launch_skinny(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K,
                          const int* a_rows, const int* group_offsets, int groups, const float* act_scale,
-                         hipStream_t stream, Picks pk = Picks{}, int act = ACT_SILU) {
+                         hipStream_t stream, Picks pk = Picks{}, GatedAct act = GatedAct{ACT_SILU, 0.f}) {
   dim3 grid(ceil_div(ACT ? N / 2 : N, 16 * (ACT ? R / 2 : R)), groups > 0 ? groups : 1), block(NW * kWave);
   const int* go = groups > 0 ? group_offsets : nullptr;
   if (out_dtype == DT_F32)

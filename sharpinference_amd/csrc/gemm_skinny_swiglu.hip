@@ -11,8 +11,9 @@
 SHARPI_EXPORT int sharpi_gemm_skinny_swiglu(const void* x, const void* W, void* out, int M, int N, int K,
                                             const int* a_rows, const int* group_offsets, int groups,
                                             const float* act_scale, int R, int NW, int packed, int row_blocks,
-                                            int act, hipStream_t stream) {
+                                            int act_code, float act_limit, hipStream_t stream) {
   if (M <= 0) return SHARPI_OK;
+  const GatedAct act{act_code, act_limit};
   if (N <= 0 || (N & 7) || K <= 0 || (K & 127) || groups <= 0 || groups > 65535 || !act_known(act)) return SHARPI_ERR_ARG;
   if (group_offsets == nullptr) return SHARPI_ERR_ARG;
   if (packed && (N & 31)) return SHARPI_ERR_ARG;
@@ -35,7 +36,7 @@ SHARPI_EXPORT int sharpi_gemm_skinny_swiglu(const void* x, const void* W, void* 
 
 // The picked form's SwiGLU half (see sharpi_gemm_skinny_picked): the arguments are checked there.
 int skinny_picked_swiglu(const void* x, const void* W, void* out, int M, int N, int K, const Picks& pk, int groups, int R,
-                         int NW, int packed, int act, hipStream_t stream) {
+                         int NW, int packed, GatedAct act, hipStream_t stream) {
   const int MB = pk.n_pairs <= 16 ? 1 : pk.n_pairs <= 32 ? 2 : 4;
 #define SKP1(RR, WW, MBV, PK) \
   return launch_skinny<RR, MBV, WW, true, PK>(x, W, out, DT_BF16, M, N, K, nullptr, pk.ids, groups, nullptr, stream, pk, act)

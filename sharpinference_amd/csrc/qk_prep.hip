@@ -4,7 +4,13 @@
 // shared by the heads; or over the whole projection, one weight per channel), rotary positions on
 // the first r elements of every head (pairs interleaved or split in halves, cos and sin times a
 // magnitude), and the write of keys and values into the paged cache.  Values may be the keys as
-// they were before norm and rotation (a layer without a value projection).
+// they were before norm and rotation (a layer without a value projection).  Further options: a bias
+// per projected channel (float, added to the row as it is gathered; not together with a
+// convolution), a query temperature 1 + c ln(floor((p + 1) / f) + 1) on q, and heads that hold
+// several score maps side by side (`maps`): norm weights and cache rows stay per head, the rotation
+// works on each map's own leading elements, and the queries leave expanded, one row of the head's
+// width per (head, map) with that map's elements in their place and zeros elsewhere, so that an
+// attention kernel over keys of the head's width computes each map's scores on its own.
 //
 // One block per token, or, in steps of few tokens, one per (token, kv head): the block then takes
 // that kv head's key and value and the query heads that read it, so that a decode step still fills
@@ -46,6 +52,10 @@ struct PrepArgs {
   const int* slot_mapping; // [T], -1: store nothing
   int page_size;
   int parts;               // blocks a token: 1, or nkv (a kv head and its query heads each)
+  const float* bias;       // [q + k + v channels] or null
+  int temp_on;             // query temperature
+  float temp_floor, temp_scale;
+  int maps;                // score maps a head (1: the plain layout of q_out; > 1: q_out [T, nh * maps * hd], expanded)
 };
 
 template <typename T>
@@ -94,7 +104,8 @@ __global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
     for (int c = threadIdx.x; c < C; c += kPrepThreads) {
       if (!mine(c)) continue;
       const int col = c < qn ? a.q_off + c : c < qn + kn ? a.k_off + (c - qn) : a.v_off + (c - qn - kn);
-      row[c] = to_f32<T>(proj[(size_t)t * a.stride + col]);
+      const float u = to_f32<T>(proj[(size_t)t * a.stride + col]);
+      row[c] = a.bias ? u + a.bias[c] : u;
     }
   }
   __syncthreads();
@@ -136,11 +147,14 @@ __global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
 
   // 4. norm, rotation, and out: a thread takes a pair of a head (or two elements that do not turn)
   const float pos = (float)a.positions[t];
-  const int half_hd = a.hd / 2, half_r = a.rotary_dim / 2;
-  T* qo = (T*)a.q_out + (size_t)t * qn;
+  const int sd = a.hd / a.maps;                          // width of one map of a head (the head's, with one map)
+  const int half_hd = a.hd / 2, half_sd = sd / 2, half_r = a.rotary_dim / 2;
+  T* qo = (T*)a.q_out + (size_t)t * qn * a.maps;
   T* kc = (T*)a.k_cache;
+  const float temp = a.temp_on ? 1.0f + a.temp_scale * logf(floorf((pos + 1.0f) / a.temp_floor) + 1.0f) : 1.0f;
   for (int i = threadIdx.x; i < heads * half_hd; i += kPrepThreads) {
-    const int h = i / half_hd, pi = i % half_hd;
+    const int hs = i / half_sd, pi = i % half_sd;         // (head, map) and the pair inside the map
+    const int h = hs / a.maps, mp = hs % a.maps, at = mp * sd;
     if (!all && !(h < a.nh ? (h >= qh0 && h < qh1) : (h - a.nh >= kh0 && h - a.nh < kh1))) continue;
     int d0, d1;
     bool turns;
@@ -154,6 +168,8 @@ __global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
       d1 = d0 + 1;
     }
     const bool is_q = h < a.nh;
+    d0 += at;
+    d1 += at;
     float x0 = row[(size_t)h * a.hd + d0], x1 = row[(size_t)h * a.hd + d1];
     if (a.norm_mode != NORM_NONE) {
       const float* w = is_q ? a.q_norm_w : a.k_norm_w;
@@ -169,8 +185,20 @@ __global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
       x1 = y1;
     }
     if (is_q) {
-      qo[(size_t)h * a.hd + d0] = from_f32<T>(x0);
-      qo[(size_t)h * a.hd + d1] = from_f32<T>(x1);
+      x0 *= temp;
+      x1 *= temp;
+      if (a.maps == 1) {
+        qo[(size_t)h * a.hd + d0] = from_f32<T>(x0);
+        qo[(size_t)h * a.hd + d1] = from_f32<T>(x1);
+      } else {
+        // the (head, map)'s own row of the head's width: the map's elements in place, zeros in the other maps' places
+        T* qr = qo + ((size_t)h * a.maps + mp) * a.hd;
+        for (int mm = 0; mm < a.maps; ++mm) {
+          const int sh = (mm - mp) * sd;
+          qr[d0 + sh] = from_f32<T>(mm == mp ? x0 : 0.f);
+          qr[d1 + sh] = from_f32<T>(mm == mp ? x1 : 0.f);
+        }
+      }
     } else if (slot >= 0) {
       const int page = slot / a.page_size, off = slot % a.page_size;
       T* kr = kc + (((size_t)page * a.nkv + (h - a.nh)) * a.page_size + off) * a.hd;
@@ -207,14 +235,20 @@ __global__ void conv_tail_kernel(const T* __restrict__ proj, int stride, int q_o
 // [slots, taps - 1, channels].  norm_mode 0 none / 1 per head (weights [hd]) / 2 whole projection
 // (weights [nh*hd], [nkv*hd]).  inv_freq float [rotary_dim / 2] or null.  Caches K [pages, nkv,
 // page_size, hd], V [pages, nkv, vd, page_size]; slot_mapping null or -1: nothing is stored.
+// bias float [q + k + v channels] or null (only without a convolution); temp_on: q times
+// 1 + temp_scale ln(floor((pos + 1) / temp_floor) + 1); maps > 1: hd is the width of a head's maps
+// together, rotary_dim <= hd / maps, and q_out is [T, nh * maps * hd].
 SHARPI_EXPORT int sharpi_qk_prep(const void* proj, int dtype, int stride, int q_off, int k_off, int v_off, int n_tokens,
                                  int n_entries, int nh, int nkv, int hd, int vd, const float* conv_w, int taps, float* tail,
                                  const int* state_slots, const int* entry_of_token, const int* cu_tokens,
                                  const int* positions, int norm_mode, const float* q_norm_w, const float* k_norm_w,
                                  float eps, const float* inv_freq, int rotary_dim, int half_split, float magnitude,
                                  void* q_out, void* k_cache, void* v_cache, const int* slot_mapping, int page_size,
-                                 int update_tail, hipStream_t stream) {
+                                 int update_tail, const float* bias, int temp_on, float temp_floor, float temp_scale,
+                                 int maps, hipStream_t stream) {
   if (n_tokens <= 0) return SHARPI_OK;
+  if (maps < 1 || hd % (2 * maps) || rotary_dim > hd / maps) return SHARPI_ERR_ARG;
+  if ((bias && taps > 0) || (temp_on && !(temp_floor > 0.f))) return SHARPI_ERR_ARG;
   if (nh <= 0 || nkv <= 0 || hd <= 0 || hd % 2 || vd <= 0 || nh + nkv > kPrepMaxHeads) return SHARPI_ERR_ARG;
   if (taps < 0 || taps == 1 || taps > kPrepMaxTaps || (taps > 0 && (!conv_w || !tail || !state_slots || !cu_tokens || !entry_of_token)))
     return SHARPI_ERR_ARG;
@@ -228,7 +262,8 @@ SHARPI_EXPORT int sharpi_qk_prep(const void* proj, int dtype, int stride, int q_
   const int parts = (n_tokens <= kPrepSplitTokens && nkv > 1 && nkv <= 65535 && nh % nkv == 0) ? nkv : 1;
   PrepArgs a{proj, stride, q_off, k_off, v_off, nh, nkv, hd, vd, conv_w, taps, tail, state_slots, entry_of_token,
              cu_tokens, positions, norm_mode, q_norm_w, k_norm_w, eps, rotary_dim > 0 ? inv_freq : nullptr, rotary_dim,
-             half_split, magnitude, q_out, k_cache, v_cache, slot_mapping, page_size, parts};
+             half_split, magnitude, q_out, k_cache, v_cache, slot_mapping, page_size, parts, bias, temp_on, temp_floor,
+             temp_scale, maps};
   dim3 pgrid(n_tokens, parts);
   if (dtype == DT_F32) qk_prep_kernel<float><<<pgrid, kPrepThreads, lds, stream>>>(a);
   else if (dtype == DT_BF16) qk_prep_kernel<bf16_t><<<pgrid, kPrepThreads, lds, stream>>>(a);

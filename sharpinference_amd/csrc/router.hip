@@ -30,7 +30,9 @@ constexpr int kGroupTop = 2;
 __device__ void gate_and_pick(float* g, int n_experts, int k, int gate, int renorm, int* ids, float* w,
                               float* gate_out, float* choice = nullptr, const float* corr = nullptr,
                               int n_groups = 1, int keep = 1) {
-  if (gate == 0) {
+  if (gate == 2) {
+    // the logits themselves rank the experts; the picks' weights are the softmax over the picked logits alone
+  } else if (gate == 0) {
     for (int e = 0; e < n_experts; ++e) g[e] = 1.0f / (1.0f + expf(-g[e]));
   } else {
     float mx = g[0];
@@ -100,6 +102,18 @@ __device__ void gate_and_pick(float* g, int n_experts, int k, int gate, int reno
     w[j] = g[best];
     wsum += g[best];
   }
+  if (gate == 2) {
+    float mx = w[0];
+    for (int j = 1; j < k; ++j) mx = fmaxf(mx, w[j]);
+    float sum = 0.f;
+    for (int j = 0; j < k; ++j) {
+      w[j] = expf(w[j] - mx);
+      sum += w[j];
+    }
+    const float inv = 1.0f / sum;
+    for (int j = 0; j < k; ++j) w[j] *= inv;
+    return;
+  }
   if (renorm && k > 1 && wsum > 0.f)
     for (int j = 0; j < k; ++j) w[j] /= wsum;
 }
@@ -163,7 +177,7 @@ __global__ __launch_bounds__(1024) void router_topk_kernel(const T* __restrict__
                                                            float* __restrict__ gate_out, int n_tokens, int hidden,
                                                            int n_experts, int k, int gate, int renorm,
                                                            const float* __restrict__ corr, int n_groups, int keep,
-                                                           int split_choice) {
+                                                           int split_choice, const float* __restrict__ bias) {
   // TT tokens per block: a router row is fetched once for all of them.
   __shared__ float g[TT][kMaxExperts];
   extern __shared__ float choice_s[];        // [TT][n_experts + n_groups] when the choice has scores of its own
@@ -179,7 +193,7 @@ __global__ __launch_bounds__(1024) void router_topk_kernel(const T* __restrict__
     wave_dot_rows<T, TW, TT>(xr, wr + (size_t)e * hidden, hidden, lane, v);
     if (lane == 0) {
 #pragma unroll
-      for (int i = 0; i < TT; ++i) g[i][e] = v[i];
+      for (int i = 0; i < TT; ++i) g[i][e] = bias ? v[i] + bias[e] : v[i];
     }
   }
   __syncthreads();
@@ -279,13 +293,15 @@ SHARPI_EXPORT int sharpi_add_rmsnorm_router(float* h, const void* delta, const v
 
 // corr (float [n_experts] or null): added to the gate values for the choice only.  n_groups, keep:
 // picks come from the `keep` best of n_groups equal groups of neighbouring experts (1, 1: no groups).
+// bias (float [n_experts] or null): added to the logits.  gate 0: sigmoid; 1: softmax over all experts;
+// 2: the largest logits are picked and their weights are the softmax over the picked logits alone.
 SHARPI_EXPORT int sharpi_router_topk(const void* x, int x_dtype, const void* wr, int w_dtype, int* topk_ids,
                                      float* topk_w, float* gate_out, int n_tokens, int hidden, int n_experts,
                                      int k, int gate, int renorm, const float* corr, int n_groups, int keep,
-                                     hipStream_t stream) {
+                                     const float* bias, hipStream_t stream) {
   if (n_tokens <= 0) return SHARPI_OK;
   if (hidden <= 0 || n_experts <= 0 || n_experts > kMaxExperts || k <= 0 || k > n_experts) return SHARPI_ERR_ARG;
-  if (gate < 0 || gate > 1) return SHARPI_ERR_ARG;
+  if (gate < 0 || gate > 2) return SHARPI_ERR_ARG;
   if (n_groups < 1 || keep < 1 || keep > n_groups || n_experts % n_groups != 0 || k > keep * (n_experts / n_groups)) return SHARPI_ERR_ARG;
   const int split_choice = corr != nullptr || keep < n_groups;
   // one wave per expert at a time: enough waves for the experts, at most 16; with many tokens four
@@ -298,11 +314,11 @@ SHARPI_EXPORT int sharpi_router_topk(const void* x, int x_dtype, const void* wr,
     if (tt == 4)                                                                                                 \
       router_topk_kernel<TX, TWT, 4><<<grid, block, lds, stream>>>((const TX*)x, (const TWT*)wr, topk_ids, topk_w, \
                                                                  gate_out, n_tokens, hidden, n_experts, k, gate, \
-                                                                 renorm, corr, n_groups, keep, split_choice);    \
+                                                                 renorm, corr, n_groups, keep, split_choice, bias);    \
     else                                                                                                         \
       router_topk_kernel<TX, TWT, 1><<<grid, block, lds, stream>>>((const TX*)x, (const TWT*)wr, topk_ids, topk_w, \
                                                                  gate_out, n_tokens, hidden, n_experts, k, gate, \
-                                                                 renorm, corr, n_groups, keep, split_choice);    \
+                                                                 renorm, corr, n_groups, keep, split_choice, bias);    \
   } while (0)
   if (x_dtype == DT_F32 && w_dtype == DT_F32) ROUTER_LAUNCH(float, float);
   else if (x_dtype == DT_BF16 && w_dtype == DT_BF16) ROUTER_LAUNCH(bf16_t, bf16_t);

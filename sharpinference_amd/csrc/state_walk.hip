@@ -10,6 +10,9 @@
 //   WALK_STATE_SPACE (a selective state space): dt = softplus(x_dt + bias_dt), a_t = exp(-exp(A_log) dt),
 //       b_t = dt; k and q are the state's input and output vectors, shared by the heads of a group; the
 //       output is o_t + D v_t.
+//   WALK_FIXED_DECAY (retention): a_t is one stored number per head and b_t one number for the layer (the
+//       keys' scale); q and k are first turned by rotary positions on their leading elements (pairs (i, i +
+//       r/2), angle = position x frequency, in float, on the staged floats), the output is o_t itself.
 // Everything but the reading of q, k, v is float: the gates, their logarithms and exponentials, the
 // running maximum, the state, the sums.
 //
@@ -36,7 +39,7 @@
 // writes the outputs, and the entry's last segment leaves the new state in the slot.
 #include "common.h"
 
-enum : int { WALK_EXP_GATES = 0, WALK_STATE_SPACE = 1 };
+enum : int { WALK_EXP_GATES = 0, WALK_STATE_SPACE = 1, WALK_FIXED_DECAY = 2 };
 enum : int { WALK_WHOLE = 0, WALK_LOCAL = 1, WALK_FINAL = 2 };
 constexpr int kWalkCols = 8;       // value columns of a block
 constexpr int kWalkChunk = 8;      // tokens staged at a time
@@ -78,7 +81,8 @@ __global__ __launch_bounds__(kWave) void state_walk_kernel(
     const float* __restrict__ p2, float cap, float q_scale, float* __restrict__ state,
     const int* __restrict__ state_slots, const int* __restrict__ cu_tokens, float* __restrict__ out, int nh, int dk,
     int dv, int ncb, int vec, const int* __restrict__ segs, float* __restrict__ seg_local,
-    const float* __restrict__ seg_start, float* __restrict__ seg_decay) {
+    const float* __restrict__ seg_start, float* __restrict__ seg_decay, const int* __restrict__ positions,
+    const float* __restrict__ inv_freq, int rot_dim, float k_scale) {
   constexpr int DKP = RPL * 8;
   constexpr int V = 16 / (int)sizeof(T);            // elements of a 16-byte load
   __shared__ __attribute__((aligned(16))) float q_s[PHASE == WALK_LOCAL ? 1 : kWalkChunk][DKP];     // (no outputs, no queries)
@@ -132,6 +136,9 @@ __global__ __launch_bounds__(kWave) void state_walk_kernel(
   if (MODE == WALK_EXP_GATES) {
     par0 = p0[h];
     par1 = p1[h];
+  } else if (MODE == WALK_FIXED_DECAY) {
+    par0 = p0[h];                 // the head's decay
+    par1 = logf(par0);
   } else {
     par0 = p0[h];                 // dt bias
     par1 = -expf(p1[h]);          // -exp(A_log)
@@ -179,7 +186,32 @@ __global__ __launch_bounds__(kWave) void state_walk_kernel(
       const int cc = cb * kWalkCols + jj;
       v_s[tt][jj] = (tt < nt && cc < dv) ? to_f32<T>(proj[(size_t)(t0 + tt) * stride + v_off + (size_t)h * dv + cc]) : 0.f;
     }
-    {
+    if (MODE == WALK_FIXED_DECAY) {
+      if (lane < nt) {
+        a_s[lane] = par0;
+        b_s[lane] = k_scale;
+      }
+      if (PHASE == WALK_LOCAL) log_decay += (float)nt * par1;
+      if (rot_dim > 0) {
+        // rotary positions on the staged floats: element i of a head with element i + rot_dim / 2
+        __syncthreads();
+        const int half = rot_dim >> 1;
+        for (int idx = lane; idx < nt * half; idx += kWave) {
+          const int tt = idx / half, i = idx % half;
+          const float ang = (float)positions[t0 + tt] * inv_freq[i];
+          const float cs = cosf(ang), sn = sinf(ang);
+          const int at0 = staged_at<RPL>(i), at1 = staged_at<RPL>(i + half);
+          const float ku = k_s[tt][at0], kv = k_s[tt][at1];
+          k_s[tt][at0] = ku * cs - kv * sn;
+          k_s[tt][at1] = kv * cs + ku * sn;
+          if (PHASE != WALK_LOCAL) {
+            const float qu = q_s[tt][at0], qv = q_s[tt][at1];
+            q_s[tt][at0] = qu * cs - qv * sn;
+            q_s[tt][at1] = qv * cs + qu * sn;
+          }
+        }
+      }
+    } else {
       const bool live = lane < nt;
       const float* grow = gates + (size_t)(t0 + (live ? lane : 0)) * gate_stride;
       if (MODE == WALK_EXP_GATES) {
@@ -258,6 +290,8 @@ __global__ __launch_bounds__(kWave) void state_walk_kernel(
         nq += __shfl_xor(nq, 16, kWave);
         nq += __shfl_xor(nq, 32, kWave);
         y = acc / (fmaxf(fabsf(nq), e_s[tt]) + kWalkFloor);
+      } else if (MODE == WALK_FIXED_DECAY) {
+        y = acc;
       } else {
         y = fmaf(par2, vj, acc);
       }
@@ -345,6 +379,7 @@ struct WalkArgs {
   float cap, q_scale; float* state; const int *state_slots, *cu_tokens; float* out;
   int n_entries, nh, dk, dv;
   const int *segs, *ent_segs; int n_segs; float *seg_local, *seg_start, *seg_decay;
+  const int* positions; const float* inv_freq; int rot_dim; float k_scale;      // WALK_FIXED_DECAY
 };
 
 template <typename T, int RPL, int MODE, int PHASE>
@@ -353,7 +388,7 @@ static void launch_walk_phase(const WalkArgs& a, int ncb, int vec, hipStream_t s
   state_walk_kernel<T, RPL, MODE, PHASE><<<grid, kWave, 0, stream>>>(
       (const T*)a.proj, a.stride, a.q_off, a.k_off, a.v_off, a.heads_per_group, a.gates, a.gate_stride, a.p0, a.p1, a.p2,
       a.cap, a.q_scale, a.state, a.state_slots, a.cu_tokens, a.out, a.nh, a.dk, a.dv, ncb, vec, a.segs, a.seg_local,
-      a.seg_start, a.seg_decay);
+      a.seg_start, a.seg_decay, a.positions, a.inv_freq, a.rot_dim, a.k_scale);
 }
 
 template <typename T, int RPL, int MODE>
@@ -390,13 +425,21 @@ static int launch_state_walk(const WalkArgs& a, hipStream_t stream) {
 static int state_walk_any(const WalkArgs& a, int dtype, int mode, hipStream_t stream) {
   if (a.n_entries <= 0) return SHARPI_OK;
   if (a.nh <= 0 || a.nh > 65535 || a.n_entries > 65535 || a.dk <= 0 || a.dk > 256 || a.dv <= 0 || a.heads_per_group <= 0) return SHARPI_ERR_ARG;
-  if (mode != WALK_EXP_GATES && mode != WALK_STATE_SPACE) return SHARPI_ERR_ARG;
-  if (!a.gates || !a.p0 || !a.p1 || (mode == WALK_STATE_SPACE && !a.p2) || (mode == WALK_EXP_GATES && !(a.cap > 0.f))) return SHARPI_ERR_ARG;
+  if (mode != WALK_EXP_GATES && mode != WALK_STATE_SPACE && mode != WALK_FIXED_DECAY) return SHARPI_ERR_ARG;
+  if (mode == WALK_FIXED_DECAY) {
+    if (!a.p0 || a.rot_dim < 0 || (a.rot_dim & 1) || a.rot_dim > a.dk || (a.rot_dim > 0 && (!a.positions || !a.inv_freq))) return SHARPI_ERR_ARG;
+  } else if (!a.gates || !a.p0 || !a.p1 || (mode == WALK_STATE_SPACE && !a.p2) || (mode == WALK_EXP_GATES && !(a.cap > 0.f))) {
+    return SHARPI_ERR_ARG;
+  }
   if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;
   if (a.segs && (!a.ent_segs || !a.seg_local || !a.seg_start || !a.seg_decay || a.n_segs < a.n_entries || a.n_segs > 65535)) return SHARPI_ERR_ARG;
   if (mode == WALK_EXP_GATES) {
     if (dtype == DT_F32) return launch_state_walk<float, WALK_EXP_GATES>(a, stream);
     return launch_state_walk<bf16_t, WALK_EXP_GATES>(a, stream);
+  }
+  if (mode == WALK_FIXED_DECAY) {
+    if (dtype == DT_F32) return launch_state_walk<float, WALK_FIXED_DECAY>(a, stream);
+    return launch_state_walk<bf16_t, WALK_FIXED_DECAY>(a, stream);
   }
   if (dtype == DT_F32) return launch_state_walk<float, WALK_STATE_SPACE>(a, stream);
   return launch_state_walk<bf16_t, WALK_STATE_SPACE>(a, stream);
@@ -405,15 +448,19 @@ static int state_walk_any(const WalkArgs& a, int dtype, int mode, hipStream_t st
 // proj [T, stride] (dtype): q and k of head h at columns q_off / k_off + (h / heads_per_group) dk, v at
 // v_off + h dv.  gates float [T, gate_stride]: WALK_EXP_GATES reads columns h (input gate) and nh + h
 // (forget gate), p0 / p1 their biases [nh], cap the gates' cap; WALK_STATE_SPACE reads column h (the
-// step size before its softplus), p0 its bias, p1 A_log, p2 D (all [nh]).  state float [slots, nh,
+// step size before its softplus), p0 its bias, p1 A_log, p2 D (all [nh]); WALK_FIXED_DECAY reads no gates:
+// p0 the heads' decays [nh], k_scale the keys' scale, and positions int [T], inv_freq float [rot_dim / 2]
+// turn the leading rot_dim elements of q and k (rot_dim 0: no rotation).  state float [slots, nh,
 // ceil(dv / 8), slice]; out float [T, nh dv].
 SHARPI_EXPORT int sharpi_state_walk(const void* proj, int dtype, int stride, int q_off, int k_off, int v_off,
                                     int heads_per_group, const float* gates, int gate_stride, const float* p0,
                                     const float* p1, const float* p2, float cap, float q_scale, int mode, float* state,
                                     const int* state_slots, const int* cu_tokens, float* out, int n_entries, int nh,
-                                    int dk, int dv, hipStream_t stream) {
+                                    int dk, int dv, const int* positions, const float* inv_freq, int rot_dim, float k_scale,
+                                    hipStream_t stream) {
   const WalkArgs a{proj, stride, q_off, k_off, v_off, heads_per_group, gates, gate_stride, p0, p1, p2, cap, q_scale, state,
-                   state_slots, cu_tokens, out, n_entries, nh, dk, dv, nullptr, nullptr, 0, nullptr, nullptr, nullptr};
+                   state_slots, cu_tokens, out, n_entries, nh, dk, dv, nullptr, nullptr, 0, nullptr, nullptr, nullptr,
+                   positions, inv_freq, rot_dim, k_scale};
   return state_walk_any(a, dtype, mode, stream);
 }
 
@@ -427,10 +474,12 @@ SHARPI_EXPORT int sharpi_state_walk_segmented(const void* proj, int dtype, int s
                                               float* state, const int* state_slots, const int* cu_tokens, float* out,
                                               int n_entries, int nh, int dk, int dv, const int* segs, const int* ent_segs,
                                               int n_segs, float* seg_local, float* seg_start, float* seg_decay,
+                                              const int* positions, const float* inv_freq, int rot_dim, float k_scale,
                                               hipStream_t stream) {
   if (!segs) return SHARPI_ERR_ARG;
   const WalkArgs a{proj, stride, q_off, k_off, v_off, heads_per_group, gates, gate_stride, p0, p1, p2, cap, q_scale, state,
-                   state_slots, cu_tokens, out, n_entries, nh, dk, dv, segs, ent_segs, n_segs, seg_local, seg_start, seg_decay};
+                   state_slots, cu_tokens, out, n_entries, nh, dk, dv, segs, ent_segs, n_segs, seg_local, seg_start, seg_decay,
+                   positions, inv_freq, rot_dim, k_scale};
   return state_walk_any(a, dtype, mode, stream);
 }
 
@@ -467,7 +516,7 @@ __global__ __launch_bounds__(256) void group_norm_gate_kernel(const float* __res
   for (int d = lane; d < gd; d += kWave) {
     float v = x[d];
     if (gate && gate_first) v *= gate_value(act, to_f32<T>(gate[d]));
-    float y = v * inv * w[(size_t)p * gd + d];
+    float y = w ? v * inv * w[(size_t)p * gd + d] : v * inv;      // (w null: a norm without a weight)
     if (gate && !gate_first) y *= gate_value(act, to_f32<T>(gate[d]));
     out[(size_t)pair * gd + d] = from_f32<T>(y);
   }

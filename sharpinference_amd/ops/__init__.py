@@ -18,8 +18,30 @@ from . import profile as _profile
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 
 WINDOW_NONE, WINDOW_CHUNK, WINDOW_SLIDING = 0, 1, 2
-ACT_SILU, ACT_GELU_TANH = 1, 2      # the gated unit's activation, as the kernels code it
-ACTIVATIONS = {"silu": ACT_SILU, "gelu_tanh": ACT_GELU_TANH}
+ACT_SILU, ACT_GELU_TANH, ACT_SWISH_CLAMP = 1, 2, 3      # the gated unit's activation, as the kernels code it
+ACTIVATIONS = {"silu": ACT_SILU, "gelu_tanh": ACT_GELU_TANH, "swish_clamp": ACT_SWISH_CLAMP}
+
+
+def gated_activation(name: str, limit: Optional[float] = None):
+    """What the kernels take as ``act`` for the gated unit `name`: its code, or for "swish_clamp" (gate
+    g = min(g, limit), up u = clamp(u, -limit, limit), result g sigmoid(1.702 g) (u + 1)) the pair
+    (code, limit)."""
+    code = ACTIVATIONS[name]
+    if code != ACT_SWISH_CLAMP:
+        if limit is not None:
+            raise ValueError(f"activation {name!r} takes no limit")
+        return code
+    if limit is None or not float(limit) > 0:
+        raise ValueError("the clamped activation needs a positive limit")
+    return (code, float(limit))
+
+
+def _act_pair(act) -> Tuple[int, float]:
+    """(code, limit) of an ``act`` argument: a code alone, or a (code, limit) pair."""
+    if isinstance(act, tuple):
+        return int(act[0]), float(act[1])
+    _need(int(act or 0) != ACT_SWISH_CLAMP, "the clamped activation comes with its limit: (code, limit)")
+    return int(act or 0), 0.0
 
 
 class KernelError(RuntimeError):
@@ -153,10 +175,11 @@ def add_rmsnorm(h: torch.Tensor, delta, weight: Optional[torch.Tensor], eps: flo
     return out
 
 
-def gated_act(gate_up: torch.Tensor, scale: Optional[torch.Tensor] = None, act: int = ACT_SILU,
+def gated_act(gate_up: torch.Tensor, scale: Optional[torch.Tensor] = None, act=ACT_SILU,
               bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """[M, 2I] (gate columns, then up columns) -> act(s*g) * (s*u) [M, I]; act: ACT_SILU or
-    ACT_GELU_TANH.  ``bias`` (float32 [2I]) is added to the gate and up columns first, in float."""
+    """[M, 2I] (gate columns, then up columns) -> act(s*g) * (s*u) [M, I]; act: ACT_SILU,
+    ACT_GELU_TANH, or (ACT_SWISH_CLAMP, limit) (see :func:`gated_activation`).  ``bias`` (float32 [2I])
+    is added to the gate and up columns first, in float."""
     _dev(gate_up, scale, bias)
     if bias is not None:
         _need(bias.dtype == torch.float32 and bias.shape == (gate_up.shape[1],), "gated_act: bias must be float32 [2I]")
@@ -165,7 +188,7 @@ def gated_act(gate_up: torch.Tensor, scale: Optional[torch.Tensor] = None, act: 
     if scale is not None:
         _need(scale.dtype == torch.float32 and scale.shape == (M,), "gated_act: scale must be float32 [M]")
     out = torch.empty(M, I2 // 2, dtype=gate_up.dtype, device=gate_up.device)
-    _run("sharpi_silu_mul", _ptr(gate_up), _ptr(scale), _ptr(out), _code(gate_up.dtype), M, I2 // 2, int(act), _ptr(bias), _stream())
+    _run("sharpi_silu_mul", _ptr(gate_up), _ptr(scale), _ptr(out), _code(gate_up.dtype), M, I2 // 2, *_act_pair(act), _ptr(bias), _stream())
     return out
 
 
@@ -736,7 +759,7 @@ def gemm_skinny(x: torch.Tensor, w, out_dtype: torch.dtype, a_rows: Optional[tor
 
 def gemm_skinny_swiglu(x: torch.Tensor, w, offsets: torch.Tensor, a_rows: Optional[torch.Tensor],
                        n_rows: int, scale: Optional[torch.Tensor], R: Optional[int] = None,
-                       NW: Optional[int] = None, group_rows: Optional[int] = None, act: int = ACT_SILU) -> torch.Tensor:
+                       NW: Optional[int] = None, group_rows: Optional[int] = None, act=ACT_SILU) -> torch.Tensor:
     """Per expert, silu(s g) * (s u) with (g | u) = x @ w[e]^T rounded to bfloat16, w [E, 2I, K]
     holding gate rows then up rows: the product and the activation in one kernel, for at most
     64 rows.  Returns [n_rows, I] bfloat16."""
@@ -762,7 +785,7 @@ def gemm_skinny_swiglu(x: torch.Tensor, w, offsets: torch.Tensor, a_rows: Option
     pr, pw = skinny_plan(N, K, _row_blocks(group_rows), E, act=True)
     out = torch.empty(M, N // 2, dtype=torch.bfloat16, device=x.device)
     _run("sharpi_gemm_skinny_swiglu", _ptr(x), _ptr(w), _ptr(out), M, N, K, _ptr(a_rows), _ptr(offsets), E,
-         _ptr(scale), R or pr, NW or pw, 1 if packed else 0, _row_blocks(group_rows), int(act), _stream())
+         _ptr(scale), R or pr, NW or pw, 1 if packed else 0, _row_blocks(group_rows), *_act_pair(act), _stream())
     return out
 
 
@@ -795,7 +818,7 @@ def gemm_skinny_picked(x: torch.Tensor, w, ids: torch.Tensor, wts: Optional[torc
     the result's row order.  act (True: SiLU; or an activation's code; False: none): w holds gate
     rows then up rows and the result is act(s g) * (s u) [rows, N/2] with s the pair's weight (wts;
     1 for the shared rows)."""
-    act = ACT_SILU if act is True else int(act or 0)
+    act, act_limit = _act_pair(ACT_SILU if act is True else act)
     w, packed = _unwrap(w)
     _dev(x, w, ids, wts)
     _i32(ids, "ids")
@@ -818,7 +841,7 @@ def gemm_skinny_picked(x: torch.Tensor, w, ids: torch.Tensor, wts: Optional[torc
     pr, pw = skinny_plan(N, K, 1 if T * k <= 16 else 2 if T * k <= 32 else 4, min(E, T * k) + (1 if shared else 0), bool(act))
     out = torch.empty(rows, N // 2 if act else N, dtype=out_dtype, device=x.device)
     _run("sharpi_gemm_skinny_picked", _ptr(x), _ptr(w), _ptr(out), _code(out_dtype), N, K, _ptr(ids), _ptr(wts), T * k, k, E,
-         1 if shared else 0, 1 if gather else 0, act, pr, pw, 1 if packed else 0, _stream())
+         1 if shared else 0, 1 if gather else 0, act, act_limit, pr, pw, 1 if packed else 0, _stream())
     return out
 
 
@@ -882,22 +905,27 @@ def grouped_gemm(x: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, a_rows
 
 
 # ---------------------------------------------------------------------------
-GATE_SIGMOID, GATE_SOFTMAX = 0, 1
+GATE_SIGMOID, GATE_SOFTMAX, GATE_SOFTMAX_PICKED = 0, 1, 2
 
 
 def router_topk(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGMOID, renorm: bool = False,
                 want_gates: bool = False, correction: Optional[torch.Tensor] = None, n_groups: int = 1,
-                keep_groups: int = 1):
-    """Router logits in float, gate, k picks (lowest index wins a tie).
+                keep_groups: int = 1, bias: Optional[torch.Tensor] = None):
+    """Router logits in float (plus ``bias``, float32 [E], where given), gate, k picks (lowest index
+    wins a tie).  Gates: sigmoid, softmax over all experts, or GATE_SOFTMAX_PICKED: the largest logits are
+    picked and the weights are the softmax over the picked logits alone (the gate values handed
+    out are then the logits).
     Returns ids int32 [T, k], weights float32 [T, k] (and the gate values [T, E] if asked).
     ``correction`` (float32 [E]) is added to the gate values for the choice only: the weights stay
     the gate values.  With ``n_groups`` > ``keep_groups`` the experts form n_groups equal groups of
     neighbours and only those of the keep_groups best groups can be picked (a group's rank: the sum
     of its two largest choice scores)."""
-    _dev(x, wr, correction)
+    _dev(x, wr, correction, bias)
     _need(x.dim() == 2 and wr.dim() == 2 and x.shape[1] == wr.shape[1], "router: x [T, H], wr [E, H]")
     T, H = x.shape
     E = wr.shape[0]
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (E,), "router: bias must be float32 [E]")
     if correction is not None:
         _need(correction.dtype == torch.float32 and correction.shape == (E,), "router: correction must be float32 [E]")
     _need(1 <= keep_groups <= n_groups and E % n_groups == 0 and k <= keep_groups * (E // n_groups),
@@ -906,7 +934,7 @@ def router_topk(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGM
     wts = torch.empty(T, k, dtype=torch.float32, device=x.device)
     gates = torch.empty(T, E, dtype=torch.float32, device=x.device) if want_gates else None
     _run("sharpi_router_topk", _ptr(x), _code(x.dtype), _ptr(wr), _code(wr.dtype), _ptr(ids), _ptr(wts), _ptr(gates),
-         T, H, E, k, gate, 1 if renorm else 0, _ptr(correction), int(n_groups), int(keep_groups), _stream())
+         T, H, E, k, gate, 1 if renorm else 0, _ptr(correction), int(n_groups), int(keep_groups), _ptr(bias), _stream())
     return (ids, wts, gates) if want_gates else (ids, wts)
 
 
@@ -997,9 +1025,10 @@ def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int, shared_gro
 
 def route(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGMOID, renorm: bool = False,
           shared_group: bool = False, correction: Optional[torch.Tensor] = None, n_groups: int = 1,
-          keep_groups: int = 1):
+          keep_groups: int = 1, bias: Optional[torch.Tensor] = None):
     """router_topk then moe_permute: (ids, weights, Routing)."""
-    ids, wts = router_topk(x, wr, k, gate, renorm, correction=correction, n_groups=n_groups, keep_groups=keep_groups)
+    ids, wts = router_topk(x, wr, k, gate, renorm, correction=correction, n_groups=n_groups, keep_groups=keep_groups,
+                           bias=bias)
     return ids, wts, moe_permute(ids, wts, wr.shape[0], shared_group)
 
 
@@ -1026,7 +1055,7 @@ def gemm_grouped(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch
 
 
 def gemm_grouped_swiglu(x: torch.Tensor, w, rt: Routing, scale: Optional[torch.Tensor], gather: bool = True,
-                        act: int = ACT_SILU, max_blocks: int = 0) -> torch.Tensor:
+                        act=ACT_SILU, max_blocks: int = 0) -> torch.Tensor:
     """Per group, act(s g) * (s u) with (g | u) = x @ w[e]^T rounded to bfloat16, for many rows: the
     grouped product with the activation (ACT_SILU, ACT_GELU_TANH) in its epilogue.  gather: x rows are read through the
     routing's token list (the order inside a group is whatever the routing kernel made it);
@@ -1045,7 +1074,7 @@ def gemm_grouped_swiglu(x: torch.Tensor, w, rt: Routing, scale: Optional[torch.T
     out = torch.empty(rt.n_rows, N // 2, dtype=torch.bfloat16, device=x.device)
     _run("sharpi_gemm_grouped_swiglu", _ptr(x), x.shape[0], _ptr(w), _ptr(out), rt.n_rows, N, K,
          _ptr(rt.sorted_token) if gather else None, _ptr(rt.offsets), _ptr(rt.plan), rt.n_groups, _ptr(scale), 1 if packed else 0,
-         int(act), int(max_blocks), _stream())
+         *_act_pair(act), int(max_blocks), _stream())
     return out
 
 
@@ -1148,15 +1177,26 @@ def qk_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: Optional[int], nh
             norm_mode: int = NORM_NONE, q_norm_w: Optional[torch.Tensor] = None, k_norm_w: Optional[torch.Tensor] = None,
             eps: float = 1e-6, inv_freq: Optional[torch.Tensor] = None, pair_layout: int = PAIRS_INTERLEAVED,
             magnitude: float = 1.0, conv_w: Optional[torch.Tensor] = None, tail: Optional[torch.Tensor] = None,
-            update_tail: bool = True) -> torch.Tensor:
+            update_tail: bool = True, bias: Optional[torch.Tensor] = None,
+            temperature: Optional[Tuple[float, float]] = None, maps: int = 1) -> torch.Tensor:
     """From a step's projections proj [T, N] (q at columns q_off.., k at k_off.., v at v_off.., or
     v_off None: the values are the keys before norm and rotation): optional short causal
     convolution over time on every channel (conv_w float32 [channels, taps]; tail float32 [slots,
     taps - 1, channels] carries each request's last projected rows from step to step and is brought
     up to date unless update_tail is False), RMS norm of q and k with learned weights (per head, or
     over the whole projection), rotary positions (cos and sin times `magnitude`), keys and values
-    into the cache at slot_mapping (None: nothing is stored).  Returns q [T, nh*hd]."""
-    _dev(proj, k_cache, v_cache, slot_mapping, q_norm_w, k_norm_w, inv_freq, conv_w, tail)
+    into the cache at slot_mapping (None: nothing is stored).  Returns q [T, nh*hd].
+
+    ``bias`` (float32, one value per channel of q, k and v; only without a convolution) is added to the
+    row as it is read.  ``temperature`` = (floor_scale, attn_scale) multiplies q by
+    1 + attn_scale * ln(floor((pos + 1) / floor_scale) + 1).  ``maps`` > 1: a head holds that many score
+    maps side by side (hd is their width together; rotary_dim at most hd / maps, applied to each map's
+    own leading elements), and q comes back expanded, [T, nh * maps * hd]: one row of the head's width
+    per (head, map), the map's elements in their place and zeros elsewhere, so that attention over
+    nh * maps query heads and keys of width hd computes every map's scores on its own."""
+    _dev(proj, k_cache, v_cache, slot_mapping, q_norm_w, k_norm_w, inv_freq, conv_w, tail, bias)
+    maps = int(maps)
+    _need(maps >= 1 and hd % (2 * maps) == 0, "qk_prep: a head must split into its maps, each of even width")
     _i32(slot_mapping, "slot_mapping")
     T, N = proj.shape
     own_v = v_off is not None
@@ -1180,6 +1220,12 @@ def qk_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: Optional[int], nh
         _need(inv_freq.dtype == torch.float32 and inv_freq.dim() == 1 and 1 <= inv_freq.shape[0] <= hd // 2,
               "qk_prep: inv_freq must be float32 [rotary_dim / 2], rotary_dim <= hd")
         rotary_dim = 2 * inv_freq.shape[0]
+        _need(rotary_dim <= hd // maps, "qk_prep: the rotated width must fit one map of a head")
+    if bias is not None:
+        _need(conv_w is None and bias.dtype == torch.float32 and bias.shape == (qn + kn + vn,),
+              "qk_prep: bias must be float32, one value per channel of q, k and v, and comes without a convolution")
+    fs, asc = temperature if temperature is not None else (1.0, 0.0)
+    _need(fs > 0, "qk_prep: the temperature's floor_scale must be positive")
     taps = 0
     if conv_w is not None:
         taps = conv_w.shape[1]
@@ -1189,13 +1235,14 @@ def qk_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: Optional[int], nh
               "qk_prep: tail must be float32 [slots, taps - 1, channels]")
         _need(ctx.state_slots.shape == (ctx.n_entries,) and ctx.cu_tokens.shape == (ctx.n_entries + 1,)
               and ctx.entry_of_token.shape == (T,), "qk_prep: the step's per-entry arrays do not fit")
-    q_out = torch.empty(T, qn, dtype=proj.dtype, device=proj.device)
+    q_out = torch.empty(T, qn * maps, dtype=proj.dtype, device=proj.device)
     page_size = k_cache.shape[2] if k_cache is not None else 0
     _run("sharpi_qk_prep", _ptr(proj), _code(proj.dtype), N, int(q_off), int(k_off), int(v_off) if own_v else -1, T,
          ctx.n_entries, nh, nkv, hd, vd, _ptr(conv_w), taps, _ptr(tail), _ptr(ctx.state_slots), _ptr(ctx.entry_of_token),
          _ptr(ctx.cu_tokens), _ptr(ctx.positions), int(norm_mode), _ptr(q_norm_w), _ptr(k_norm_w), float(eps),
          _ptr(inv_freq), rotary_dim, 1 if pair_layout == PAIRS_HALF_SPLIT else 0, float(magnitude), _ptr(q_out),
-         _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping), page_size, 1 if update_tail else 0, _stream())
+         _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping), page_size, 1 if update_tail else 0, _ptr(bias),
+         1 if temperature is not None else 0, float(fs), float(asc), maps, _stream())
     return q_out
 
 
@@ -1446,7 +1493,7 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
 
 
 def grouped_swiglu(x: torch.Tensor, w_gate_up, rt: Routing, out_dtype: torch.dtype, scaled: bool = True,
-                   act: int = ACT_SILU, max_blocks: int = 0) -> torch.Tensor:
+                   act=ACT_SILU, max_blocks: int = 0) -> torch.Tensor:
     """The experts' gate|up products of the routed tokens and their activation,
     act(s g) * (s u) with s the pick's weight (``scaled``; otherwise s = 1): [n_rows, I] in
     expert-sorted order.  On the matrix cores the activation is the product's epilogue (the
@@ -1513,7 +1560,7 @@ def measured_peaks(device="cuda:0", read_bytes: int = 4 << 30, repeats: int = 5)
 # ---------------------------------------------------------------------------
 # recurrent states with a scalar decay per (token, head); gated branches; a second input from the token
 # ---------------------------------------------------------------------------
-WALK_EXP_GATES, WALK_STATE_SPACE = 0, 1      # csrc/state_walk.hip
+WALK_EXP_GATES, WALK_STATE_SPACE, WALK_FIXED_DECAY = 0, 1, 2      # csrc/state_walk.hip
 WALK_MAX_KEY_DIM = 256
 WALK_STATE_COLS = _lib.WALK_STATE_COLS
 SHORT_CONV_MAX_TAPS = 8                       # csrc/state_walk.hip kConvMaxTaps
@@ -1550,9 +1597,9 @@ def walk_state_matrices(state: torch.Tensor, dk: int, dv: int, mode: int):
     return S, n, state[..., 0, dkp * 8 + dkp].contiguous()
 
 
-def state_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, heads_per_group: int, gates: torch.Tensor,
+def state_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, heads_per_group: int, gates: Optional[torch.Tensor],
                params, cap: float, q_scale: float, mode: int, state: torch.Tensor, ctx, nh: int, dk: int, dv: int,
-               segments=None) -> torch.Tensor:
+               segments=None, inv_freq: Optional[torch.Tensor] = None, k_scale: float = 1.0) -> torch.Tensor:
     """The recurrence S_t = a_t S_(t-1) + b_t k_t v_t^T, o_t = S_t^T q_t per head with one decay a_t and one
     input weight b_t per (token, head), token by token along every entry of the step, from and into
     state [slots, *walk_state_shape(nh, dk, dv, mode)] (float32) at the entries' state slots.  q and k of
@@ -1564,24 +1611,38 @@ def state_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, heads_per
       maximum m (starting at 0) keeps the exponentials in range, a normaliser vector n moves beside S,
       and the result is o / (max(|n . q|, exp(-m)) + 1e-6);
     * WALK_STATE_SPACE: gates column h is the step size before its softplus, params (its bias, A_log, D);
-      a = exp(-exp(A_log) dt), b = dt, and the result is o + D v.
+      a = exp(-exp(A_log) dt), b = dt, and the result is o + D v;
+    * WALK_FIXED_DECAY: no gates (``gates`` None); params (the heads' decays,): a = decay[h], b = ``k_scale``
+      (the keys' scale), and, with ``inv_freq`` (float32 [r / 2]), the leading r elements of every q and k head
+      are first turned by rotary positions, element i with element i + r/2 by the angle position x
+      inv_freq[i], in float; the result is o.
 
     ``segments`` = (segs, ent_segs) on the device (see :func:`gla_segments`): long entries are then walked
     segment by segment side by side.  A stretch of tokens acts on the state as S -> D S + L (D the product of
     its decays, one number a head; L what it makes of a zero state), so every segment is first walked from
     nothing, the true start states follow one from the other, and a second walk from those writes the
     outputs (results equal to rounding).  Returns float32 [T, nh * dv]."""
-    _dev(proj, gates, state, *params)
+    _dev(proj, gates, state, inv_freq, *params)
     T, N = proj.shape
     groups = nh // heads_per_group if heads_per_group > 0 else 0
     _need(1 <= dk <= WALK_MAX_KEY_DIM and dv >= 1 and nh >= 1 and heads_per_group >= 1 and nh % heads_per_group == 0,
           f"state_walk: key channels 1..{WALK_MAX_KEY_DIM}, heads a multiple of the heads a group")
     _need(min(q_off, k_off, v_off) >= 0 and max(q_off, k_off) + groups * dk <= N and v_off + nh * dv <= N,
           "state_walk: q, k and v columns must lie inside proj")
-    _need(mode in (WALK_EXP_GATES, WALK_STATE_SPACE), "state_walk: mode 0 (exponential gates) or 1 (state space)")
-    n_par, n_cols = (2, 2 * nh) if mode == WALK_EXP_GATES else (3, nh)
-    _need(gates.dtype == torch.float32 and gates.dim() == 2 and gates.shape[0] == T and gates.shape[1] >= n_cols,
-          f"state_walk: gates float32 [T, >= {n_cols}] wanted")
+    _need(mode in (WALK_EXP_GATES, WALK_STATE_SPACE, WALK_FIXED_DECAY),
+          "state_walk: mode 0 (exponential gates), 1 (state space) or 2 (a fixed decay per head)")
+    n_par, n_cols = (2, 2 * nh) if mode == WALK_EXP_GATES else (3, nh) if mode == WALK_STATE_SPACE else (1, 0)
+    rot_dim = 0
+    if mode == WALK_FIXED_DECAY:
+        _need(gates is None, "state_walk: a fixed decay reads no gates")
+        if inv_freq is not None:
+            _need(inv_freq.dtype == torch.float32 and inv_freq.dim() == 1 and 1 <= inv_freq.shape[0] <= dk // 2
+                  and ctx.positions.shape == (T,), "state_walk: inv_freq float32 [r / 2], r <= dk, and the step's positions [T]")
+            rot_dim = 2 * inv_freq.shape[0]
+    else:
+        _need(inv_freq is None and k_scale == 1.0, "state_walk: rotation and a key scale belong to the fixed-decay mode")
+        _need(gates.dtype == torch.float32 and gates.dim() == 2 and gates.shape[0] == T and gates.shape[1] >= n_cols,
+              f"state_walk: gates float32 [T, >= {n_cols}] wanted")
     _need(len(params) == n_par and all(p.dtype == torch.float32 and p.shape == (nh,) for p in params),
           f"state_walk: {n_par} float32 [nh] parameter vectors wanted")
     _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == walk_state_shape(nh, dk, dv, mode),
@@ -1590,6 +1651,8 @@ def state_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, heads_per
           "state_walk: the step's per-entry arrays do not fit")
     out = torch.empty(T, nh * dv, dtype=torch.float32, device=proj.device)
     p = list(params) + [None] * (3 - n_par)
+    g_stride = gates.shape[1] if gates is not None else 0
+    rot = (_ptr(ctx.positions) if rot_dim else None, _ptr(inv_freq) if rot_dim else None, rot_dim, float(k_scale))
     if segments is not None:
         segs, ent_segs = segments
         _dev(segs, ent_segs)
@@ -1603,26 +1666,27 @@ def state_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, heads_per
         seg_start = torch.empty(shape, dtype=torch.float32, device=proj.device)
         seg_decay = torch.empty(n_segs, nh, dtype=torch.float32, device=proj.device)
         _run("sharpi_state_walk_segmented", _ptr(proj), _code(proj.dtype), N, int(q_off), int(k_off), int(v_off),
-             int(heads_per_group), _ptr(gates), gates.shape[1], _ptr(p[0]), _ptr(p[1]), _ptr(p[2]), float(cap), float(q_scale),
+             int(heads_per_group), _ptr(gates), g_stride, _ptr(p[0]), _ptr(p[1]), _ptr(p[2]), float(cap), float(q_scale),
              int(mode), _ptr(state), _ptr(ctx.state_slots), _ptr(ctx.cu_tokens), _ptr(out), ctx.n_entries, nh, dk, dv,
-             _ptr(segs), _ptr(ent_segs), n_segs, _ptr(seg_local), _ptr(seg_start), _ptr(seg_decay), _stream())
+             _ptr(segs), _ptr(ent_segs), n_segs, _ptr(seg_local), _ptr(seg_start), _ptr(seg_decay), *rot, _stream())
         return out
     _run("sharpi_state_walk", _ptr(proj), _code(proj.dtype), N, int(q_off), int(k_off), int(v_off), int(heads_per_group),
-         _ptr(gates), gates.shape[1], _ptr(p[0]), _ptr(p[1]), _ptr(p[2]), float(cap), float(q_scale), int(mode), _ptr(state),
-         _ptr(ctx.state_slots), _ptr(ctx.cu_tokens), _ptr(out), ctx.n_entries, nh, dk, dv, _stream())
+         _ptr(gates), g_stride, _ptr(p[0]), _ptr(p[1]), _ptr(p[2]), float(cap), float(q_scale), int(mode), _ptr(state),
+         _ptr(ctx.state_slots), _ptr(ctx.cu_tokens), _ptr(out), ctx.n_entries, nh, dk, dv, *rot, _stream())
     return out
 
 
-def group_norm_gate(o: torch.Tensor, weight: torch.Tensor, eps: float, groups: int, out_dtype: torch.dtype,
+def group_norm_gate(o: torch.Tensor, weight: Optional[torch.Tensor], eps: float, groups: int, out_dtype: torch.dtype,
                     gate_proj: Optional[torch.Tensor] = None, gate_off: int = 0, gate_act: int = GATE_NONE,
                     gate_first: bool = False) -> torch.Tensor:
     """o float32 [T, N] in `groups` equal parts, each divided by its root mean square, times weight
-    (float32 [N]), times act(gate) (columns gate_off.. of gate_proj [T, M], of out_dtype; act GATE_SILU
+    (float32 [N]; None: no weight), times act(gate) (columns gate_off.. of gate_proj [T, M], of out_dtype; act GATE_SILU
     or GATE_SIGMOID_ACT).  ``gate_first``: the gate multiplies o before the statistics are taken."""
     _dev(o, weight, gate_proj)
     T, N = o.shape
-    _need(o.dtype == torch.float32 and groups >= 1 and N % groups == 0 and weight.dtype == torch.float32 and weight.shape == (N,),
-          "group_norm_gate: o float32 [T, N], N a multiple of the groups, weight float32 [N]")
+    _need(o.dtype == torch.float32 and groups >= 1 and N % groups == 0
+          and (weight is None or (weight.dtype == torch.float32 and weight.shape == (N,))),
+          "group_norm_gate: o float32 [T, N], N a multiple of the groups, weight float32 [N] or None")
     _need(gate_act in (GATE_NONE, GATE_SILU, GATE_SIGMOID_ACT), "group_norm_gate: gate_act 0, 1 or 2")
     stride = 0
     if gate_act != GATE_NONE:
@@ -1718,4 +1782,73 @@ def side_gate(gate: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, col_of
     out = torch.empty_like(gate)
     _run("sharpi_side_gate", _ptr(gate), _code(gate.dtype), _ptr(ids), _ptr(table), _code(table.dtype), table.shape[1],
          int(col_off), _ptr(out), T, D, _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------
+# several residual streams; the difference of two score maps
+# ---------------------------------------------------------------------------
+HYPER_MAX_STREAMS = 8                 # csrc/hyper.hip kHyperMaxStreams
+HYPER_MAX_WIDTH = 15 * 1024           # floats of a row that the kernel keeps in LDS
+
+
+def hyper_step(src: torch.Tensor, lanes: Optional[torch.Tensor], n_streams: int, delta=None,
+               mix: Optional[torch.Tensor] = None, out_w: Optional[torch.Tensor] = None, in_w: Optional[torch.Tensor] = None,
+               norm_w: Optional[torch.Tensor] = None, eps: float = 0.0, out_dtype: Optional[torch.dtype] = None,
+               rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """What lies between two sublayers of a model with S residual streams per token.  ``src``: the old
+    streams, float32 [T, S, W], or [T, W] when all S are still that one row.  With ``delta`` (the last
+    sublayer's output [T, W], a tensor or an ExpertSum) the streams are first brought up to date,
+    new[t] = sum_s mix[s, t] old[s] + out_w[t] delta (``mix`` float32 [S, S], ``out_w`` float32 [S]), and stored
+    in ``lanes`` (float32 [T, S, W]; may be ``src`` itself; None: not stored).  Then u = sum_s in_w[s] new[s]
+    (``in_w`` float32 [S]; None: the plain sum), and the result is unit_rms(u) * norm_w in ``out_dtype``,
+    or, with ``norm_w`` None, u itself in float32.  ``rows`` (int32): only those tokens are produced."""
+    lazy = delta if isinstance(delta, ExpertSum) else None
+    base = lazy.y if lazy is not None else delta
+    _dev(src, lanes, base, mix, out_w, in_w, norm_w, rows, *( [lazy.inv_pos, lazy.shared, lazy.weights] if lazy is not None else []))
+    _i32(rows, "rows")
+    S = int(n_streams)
+    _need(src.dtype == torch.float32 and src.dim() in (2, 3) and 1 <= S <= HYPER_MAX_STREAMS, "hyper_step: src float32 [T, S, W] or [T, W]")
+    T, W = src.shape[0], src.shape[-1]
+    _need(W <= HYPER_MAX_WIDTH and (src.dim() == 2 or src.shape[1] == S), "hyper_step: streams or width do not fit")
+    src_token, src_stream = (W, 0) if src.dim() == 2 else (S * W, W)
+    if lanes is not None:
+        _need(lanes.dtype == torch.float32 and tuple(lanes.shape) == (T, S, W), "hyper_step: lanes must be float32 [T, S, W]")
+    if delta is not None:
+        _need(tuple(delta.shape) == (T, W), f"hyper_step: delta {tuple(delta.shape)} vs [T, W] = {(T, W)}")
+        _need(mix is not None and out_w is not None and mix.dtype == torch.float32 and mix.shape == (S, S)
+              and out_w.dtype == torch.float32 and out_w.shape == (S,), "hyper_step: mix float32 [S, S] and out_w float32 [S] come with delta")
+    if in_w is not None:
+        _need(in_w.dtype == torch.float32 and in_w.shape == (S,), "hyper_step: in_w must be float32 [S]")
+    if norm_w is not None:
+        _need(norm_w.shape == (W,) and out_dtype is not None, "hyper_step: norm_w [W] and an out_dtype")
+    else:
+        out_dtype = torch.float32
+    n_out = T if rows is None else rows.shape[0]
+    out = torch.empty(n_out, W, dtype=out_dtype, device=src.device)
+    _run("sharpi_hyper_step", _ptr(src), src_token, src_stream, _ptr(lanes), _ptr(base), _code(base.dtype) if base is not None else 0,
+         _ptr(lazy.inv_pos) if lazy is not None else None, _ptr(lazy.shared) if lazy is not None else None,
+         _ptr(lazy.weights) if lazy is not None else None, lazy.k if lazy is not None else 0, _ptr(mix), _ptr(out_w), _ptr(in_w),
+         _ptr(norm_w), _code(norm_w.dtype) if norm_w is not None else 0, float(eps), _ptr(out), _code(out_dtype), _ptr(rows),
+         n_out, S, W, _stream())
+    return out
+
+
+def map_difference(a: torch.Tensor, n_heads: int, vd: int, lam: float, eps: float, post: float,
+                   gate_proj: Optional[torch.Tensor] = None, gate_off: int = 0) -> torch.Tensor:
+    """a [T, n_heads * 2 * vd]: per head the outputs a1, a2 of two score maps over the same values.  Returns
+    [T, n_heads * vd] = unit_rms(a1 - lam * a2) * post (the root mean square over a head's vd values, eps
+    inside the root, in float), times sigmoid of column gate_off + head of gate_proj [T, M] where given
+    (one gate number per head)."""
+    _dev(a, gate_proj)
+    T = a.shape[0]
+    _need(a.dim() == 2 and a.shape[1] == n_heads * 2 * vd, "map_difference: a must be [T, n_heads * 2 * vd]")
+    stride = 0
+    if gate_proj is not None:
+        _need(gate_proj.dtype == a.dtype and gate_proj.dim() == 2 and gate_proj.shape[0] == T and 0 <= gate_off
+              and gate_off + n_heads <= gate_proj.shape[1], "map_difference: the gates' columns must lie inside gate_proj")
+        stride = gate_proj.shape[1]
+    out = torch.empty(T, n_heads * vd, dtype=a.dtype, device=a.device)
+    _run("sharpi_map_difference", _ptr(a), _code(a.dtype), float(lam), float(eps), float(post), _ptr(gate_proj), stride,
+         int(gate_off), _ptr(out), T, n_heads, vd, _stream())
     return out

@@ -20,7 +20,7 @@ _SIGNATURES = {
     "sharpi_embed_gather": [P, P, I, P, I, I, F, P],
     "sharpi_scale_softcap": [P, c_longlong, F, F, P],
     "sharpi_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, P, P, P, I, P],
-    "sharpi_silu_mul": [P, P, P, I, I, I, I, P, P],
+    "sharpi_silu_mul": [P, P, P, I, I, I, I, F, P, P],
     "sharpi_moe_combine": [P, P, P, P, P, I, I, I, I, P],
     "sharpi_cast": [P, I, P, I, c_longlong, P],
     "sharpi_add_bias": [P, I, P, I, I, P],
@@ -33,10 +33,10 @@ _SIGNATURES = {
     "sharpi_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, F, I, I, I, I, I, I, F, I, P, P],
     "sharpi_gemm_tiled": [P, P, P, I, I, I, I, I, P, P, I, P],
     "sharpi_gemm_skinny": [P, P, P, I, I, I, I, P, P, I, I, I, I, I, P],
-    "sharpi_gemm_skinny_swiglu": [P, P, P, I, I, I, P, P, I, P, I, I, I, I, I, P],
-    "sharpi_gemm_skinny_picked": [P, P, P, I, I, I, P, P, I, I, I, I, I, I, I, I, I, P],
+    "sharpi_gemm_skinny_swiglu": [P, P, P, I, I, I, P, P, I, P, I, I, I, I, I, F, P],
+    "sharpi_gemm_skinny_picked": [P, P, P, I, I, I, P, P, I, I, I, I, I, I, F, I, I, I, P],
     "sharpi_add_rmsnorm_router": [P, P, P, I, P, I, I, F, P, I, P, P, I, I, I, I, P],
-    "sharpi_router_topk": [P, I, P, I, P, P, P, I, I, I, I, I, I, P, I, I, P],
+    "sharpi_router_topk": [P, I, P, I, P, P, P, I, I, I, I, I, I, P, I, I, P, P],
     "sharpi_norm_add": [P, P, I, P, P, I, I, I, F, P, P, I, P],
     "sharpi_latent_prep": [P, I, I, I, I, P, P, P, P, P, I, P, F, I, I, I, I, I, P],
     "sharpi_head_gemm": [P, I, I, I, P, P, I, I, P, I, I, I, I, I, P],
@@ -45,11 +45,11 @@ _SIGNATURES = {
     "sharpi_attention_latent_merge": [P, P, P, P, I, P, P, I, I, I, I, P],
     "sharpi_moe_permute": [P, P, P, P, P, P, P, I, I, I, I, I, P],
     "sharpi_gemm_grouped": [P, I, P, P, I, I, I, I, P, P, P, I, I, I, P],
-    "sharpi_gemm_grouped_swiglu": [P, I, P, P, I, I, I, P, P, P, I, P, I, I, I, P],
+    "sharpi_gemm_grouped_swiglu": [P, I, P, P, I, I, I, P, P, P, I, P, I, I, F, I, P],
     "sharpi_argmax_rows": [P, P, I, I, P],
     "sharpi_sample_rows": [P, P, P, P, P, P, P, P, I, I, P],
     "sharpi_edit_logits": [P, P, P, P, P, P, P, P, I, I, P],
-    "sharpi_qk_prep": [P, I, I, I, I, I, I, I, I, I, I, I, P, I, P, P, P, P, P, I, P, P, F, P, I, I, F, P, P, P, P, I, I, P],
+    "sharpi_qk_prep": [P, I, I, I, I, I, I, I, I, I, I, I, P, I, P, P, P, P, P, I, P, P, F, P, I, I, F, P, P, P, P, I, I, P, I, F, F, I, P],
     "sharpi_gla_walk": [P, I, I, I, I, I, P, F, P, P, P, P, I, I, I, I, I, P],
     "sharpi_gla_decays": [P, P, F, I, I, P],
     "sharpi_gla_walk_segmented": [P, I, I, I, I, I, P, F, P, P, P, P, I, I, I, I, P, P, I, P, P, P],
@@ -58,13 +58,15 @@ _SIGNATURES = {
     "sharpi_activation": [P, P, I, c_longlong, I, P],
     "sharpi_norm_mean": [P, P, I, I, P, I, I, F, P],
     "sharpi_post_pre_norm": [P, P, P, I, I, P, P, P, I, I, I, F, P],
-    "sharpi_state_walk": [P, I, I, I, I, I, I, P, I, P, P, P, F, F, I, P, P, P, P, I, I, I, I, P],
-    "sharpi_state_walk_segmented": [P, I, I, I, I, I, I, P, I, P, P, P, F, F, I, P, P, P, P, I, I, I, I, P, P, I, P, P, P, P],
+    "sharpi_state_walk": [P, I, I, I, I, I, I, P, I, P, P, P, F, F, I, P, P, P, P, I, I, I, I, P, P, I, F, P],
+    "sharpi_state_walk_segmented": [P, I, I, I, I, I, I, P, I, P, P, P, F, F, I, P, P, P, P, I, I, I, I, P, P, I, P, P, P, P, P, I, F, P],
     "sharpi_group_norm_gate": [P, P, F, P, I, I, I, I, I, P, I, I, I, P],
     "sharpi_short_conv": [P, I, I, I, P, P, I, P, P, P, P, P, I, I, I, I, P],
     "sharpi_sigmoid_gate": [P, P, I, I, I, P, I, I, P],
     "sharpi_stream_add": [P, P, P, I, I, P, I, c_longlong, P],
     "sharpi_side_gate": [P, I, P, P, I, I, I, P, I, I, P],
+    "sharpi_hyper_step": [P, c_longlong, c_longlong, P, P, I, P, P, P, I, P, P, P, P, I, F, P, I, P, I, I, I, P],
+    "sharpi_map_difference": [P, I, F, F, F, P, I, I, P, I, I, I, P],
 }
 
 # entry points that newer sources add; bound when present

@@ -79,13 +79,24 @@ class Attention(Part):
     ``sink`` [heads], float; not scaled).  ``gate``: the heads' outputs side by side are multiplied
     element by element by sigmoid(W_g x) (W_g [heads * v_head_dim, hidden], a product of the same
     input as q, k and v, made by the same launch) before the output projection.  A rotary object's
-    ``magnitude`` multiplies cos and sin.  ``names``: the tensors' names behind the layer's prefix."""
+    ``magnitude`` multiplies cos and sin.  ``names``: the tensors' names behind the layer's prefix.
+
+    ``score_maps`` m > 1 with ``difference`` c: differential attention.  Every query head and every key head
+    holds m = 2 score maps of ``head_dim`` elements side by side (q rows [head][map][head_dim], and so k); each
+    map is an attention of its own (position encoding per map, the same scale, window and softmax) over the
+    head's one set of values, and the head's output is unit_rms(a_1 - lambda a_2) * (1 - c) with
+    lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + c from four stored vectors [head_dim], one number for the
+    layer, the root mean square over the head's values with ``difference_eps`` inside the root.  The cache
+    keeps a key head's maps as one row of m * head_dim elements; queries are expanded to one such row per
+    (head, map) with zeros in the other map's place, so the attention kernels compute each map's scores
+    unchanged (csrc/qk_prep.hip, csrc/hyper.hip).  ``head_gate``: each head's output is multiplied by
+    sigmoid(W_g x)_h, one number per head (W_g [heads, hidden], made by the q|k|v launch)."""
 
     NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
              "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
              "q_norm": "q_norm.weight", "k_norm": "k_norm.weight",
              "q_conv": "q_conv.weight", "k_conv": "k_conv.weight", "v_conv": "v_conv.weight",
-             "sink": "sink", "g": "g_proj.weight"}
+             "sink": "sink", "g": "g_proj.weight", "lq1": "lq1", "lk1": "lk1", "lq2": "lq2", "lk2": "lk2"}
 
     def __init__(self, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  rotary=None, qk_norm_eps: Optional[float] = None,
@@ -93,14 +104,27 @@ class Attention(Part):
                  window: int = 0, scale: Optional[float] = None, bias: bool = False, o_bias: Optional[bool] = None,
                  v_head_dim: Optional[int] = None, qk_norm_weights: Optional[str] = None, values_from_keys: bool = False,
                  conv_taps: int = 0, softcap: float = 0.0, sink=False, names: Optional[Dict[str, str]] = None,
-                 gate: bool = False):
+                 gate: bool = False, score_maps: int = 1, difference: Optional[float] = None,
+                 difference_eps: Optional[float] = None, head_gate: bool = False):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads cannot share {num_kv_heads} kv heads")
-        prep = bool(qk_norm_weights or values_from_keys or conv_taps)
-        if head_dim % 2 or not 2 <= head_dim <= 256:      # (the rotation takes pairs; the attention kernels hold 256 elements)
-            raise ValueError(f"head_dim {head_dim} is not taken: even sizes from 2 to 256")
+        self.maps = int(score_maps)
+        if self.maps not in (1, 2) or (self.maps == 2) != (difference is not None):
+            raise ValueError("score_maps is 1, or 2 together with the difference's constant")
+        if self.maps == 2 and (difference_eps is None or not 0.0 <= float(difference) < 1.0):
+            raise ValueError("differential attention needs difference_eps and a constant in [0, 1)")
+        self.difference = float(difference) if difference is not None else 0.0
+        self.difference_eps = float(difference_eps) if difference_eps is not None else 0.0
+        self.head_gate = bool(head_gate)
+        if self.head_gate and (gate or self.maps == 1):
+            raise ValueError("a gate number per head belongs to differential attention and excludes the gate per channel")
+        prep = bool(qk_norm_weights or values_from_keys or conv_taps or self.maps > 1)
+        self.map_dim = int(head_dim)                      # width of one score map of a head
         if rotary is not None and rotary.head_dim != head_dim:
             raise ValueError("the rotary table's head_dim differs from the mixer's")
+        head_dim = int(head_dim) * self.maps              # a head as the cache and the kernels see it: its maps side by side
+        if head_dim % 2 or not 2 <= head_dim <= 256:      # (the rotation takes pairs; the attention kernels hold 256 elements)
+            raise ValueError(f"head_dim {head_dim} is not taken: even sizes from 2 to 256")
         if rotary is not None and rotary.pair_layout not in ("interleaved", "half"):
             raise ValueError(f"pair layout {rotary.pair_layout!r} is not taken by the rotation kernel")
         self.hidden, self.nh, self.nkv, self.hd = int(hidden), int(num_heads), int(num_kv_heads), int(head_dim)
@@ -130,9 +154,13 @@ class Attention(Part):
             raise ValueError("an output gate belongs to the rotate-then-norm form of the layer")
         if self.softcap < 0:
             raise ValueError("softcap must be positive (or 0 for none)")
+        if self.maps > 1 and (self.sink or self.softcap):
+            raise ValueError("differential attention comes without a sink and without a cap on the scores")
         self.prep = prep                                         # the layer takes the norm-before-rotation kernel
-        if prep and (q_temperature is not None or bias):
-            raise ValueError("query temperature and q/k/v biases belong to the rotate-then-norm form of the layer")
+        if prep and bias and conv_taps:
+            raise ValueError("q/k/v biases and a convolution behind the projections do not come together")
+        if prep and self.o_bias:
+            raise ValueError("an output bias belongs to the rotate-then-norm form of the layer")
         if prep and (self.nh + 2 * self.nkv) * max(self.hd, self.vd) > ops.QK_PREP_MAX_ROW:
             raise ValueError(f"a token's q, k and v of more than {ops.QK_PREP_MAX_ROW} channels are not taken")
         if not prep and rotary is not None and getattr(rotary, "magnitude", 1.0) != 1.0:
@@ -147,6 +175,7 @@ class Attention(Part):
         self.w_k_norm: Optional[torch.Tensor] = None
         self.w_conv: Optional[torch.Tensor] = None               # float32 [q + k + v channels, taps]
         self.w_sink: Optional[torch.Tensor] = None               # float32 [heads]
+        self.lam: float = 0.0                                    # the difference's lambda (from four stored vectors)
 
     # -- what it needs --------------------------------------------------------
     def step_planners(self):
@@ -186,6 +215,11 @@ class Attention(Part):
             specs[prefix + n["sink"]] = ParamSpec((self.nh,))
         if self.has_gate:
             specs[prefix + n["g"]] = ParamSpec((ov, self.hidden))
+        if self.head_gate:
+            specs[prefix + n["g"]] = ParamSpec((self.nh, self.hidden))
+        if self.maps > 1:
+            for key in ("lq1", "lk1", "lq2", "lk2"):
+                specs[prefix + n[key]] = ParamSpec((self.map_dim,))
         if self.conv_taps:
             specs[prefix + n["q_conv"]] = ParamSpec((q, self.conv_taps))
             specs[prefix + n["k_conv"]] = ParamSpec((kv, self.conv_taps))
@@ -196,7 +230,7 @@ class Attention(Part):
     def load(self, prefix: str, source: TensorSource) -> None:
         n = self.names
         kinds = ("q", "k") if self.values_from_keys else ("q", "k", "v")
-        parts = [source.get(prefix + n[k]) for k in kinds + (("g",) if self.has_gate else ())]
+        parts = [source.get(prefix + n[k]) for k in kinds + (("g",) if self.has_gate or self.head_gate else ())]
         dt = torch.float32 if any(p.dtype == torch.float32 for p in parts) else parts[0].dtype
         fused = torch.empty(sum(p.shape[0] for p in parts), self.hidden, dtype=dt, device=parts[0].device)
         o = 0
@@ -215,6 +249,9 @@ class Attention(Part):
             self.w_k_norm = source.get(prefix + n["k_norm"]).float().contiguous()
         if self.learned_sink:
             self.w_sink = source.get(prefix + n["sink"]).float().contiguous()
+        if self.maps > 1:
+            lq1, lk1, lq2, lk2 = (source.get(prefix + n[key]).float() for key in ("lq1", "lk1", "lq2", "lk2"))
+            self.lam = float(torch.exp((lq1 * lk1).sum()) - torch.exp((lq2 * lk2).sum()) + self.difference)
         if self.conv_taps:
             self.w_conv = torch.cat([source.get(prefix + n[k + "_conv"]).float() for k in kinds]).contiguous()
 
@@ -224,7 +261,7 @@ class Attention(Part):
         T = x.shape[0]
         width = 2 if ctx.act_dtype == torch.bfloat16 else 4
         q_dim, kv_dim = self.nh * self.hd, self.nkv * (self.hd + self.vd) // 2    # (kv_dim: the mean of a key's and a value's row)
-        g_dim = self.nh * self.vd if self.has_gate else 0
+        g_dim = self.nh * self.vd if self.has_gate else self.nh if self.head_gate else 0
         with section("qkv", nbytes=width * (q_dim + 2 * kv_dim + g_dim) * (self.hidden + T) + width * T * self.hidden,
                      flops=2.0 * T * self.hidden * (q_dim + 2 * kv_dim + g_dim)):
             qkv = ops.linear(x, self.w_qkv, ctx.act_dtype)
@@ -239,15 +276,20 @@ class Attention(Part):
                                 self.vd, ctx, cache.k, cache.v, slots, mode, self.w_q_norm, self.w_k_norm,
                                 self.qk_norm_eps or 1e-6, inv_freq, layout,
                                 getattr(self.rotary, "magnitude", 1.0) if self.rotary is not None else 1.0,
-                                self.w_conv, cache.states[0] if self.conv_taps else None, update_tail=cache.write)
+                                self.w_conv, cache.states[0] if self.conv_taps else None, update_tail=cache.write,
+                                bias=self.b_qkv, temperature=self.q_temperature, maps=self.maps)
             else:
                 q = ops.rope_kv(qkv, cache.k, cache.v, slots, ctx.positions, inv_freq, self.qk_norm_eps is not None,
                                 self.qk_norm_eps or 1e-6, self.q_temperature, self.nh, self.nkv, self.hd, layout,
                                 bias=self.b_qkv, vd=self.vd, extra_columns=g_dim)
         with section("attention", nbytes=lambda: self._keys_held(ctx) * 2 * kv_dim * width + 2 * T * q_dim * width,
                      flops=lambda: 4.0 * self._keys_read(ctx) * q_dim):
-            o = ops.attention(q, cache.k, cache.v, g, ctx, self.window_kind, self.window, self.scale, self.nh, self.nkv,
-                              self.hd, self.vd, softcap=self.softcap, sink=self.w_sink if self.learned_sink else self.sink)
+            o = ops.attention(q, cache.k, cache.v, g, ctx, self.window_kind, self.window, self.scale, self.nh * self.maps,
+                              self.nkv, self.hd, self.vd, softcap=self.softcap, sink=self.w_sink if self.learned_sink else self.sink)
+        if self.maps > 1:
+            with section("difference of the maps", nbytes=3 * width * T * self.nh * self.vd):
+                o = ops.map_difference(o, self.nh, self.vd, self.lam, self.difference_eps, 1.0 - self.difference,
+                                       qkv if self.head_gate else None, qkv.shape[1] - g_dim)
         if self.has_gate:
             with section("output gate", nbytes=3 * width * T * g_dim):
                 o = ops.sigmoid_gate(o, qkv, qkv.shape[1] - g_dim)

@@ -130,6 +130,10 @@ class ResidualStream:
         self.pending_norm = None   # a norm that sits on `pending` before it is added (h += norm(pending)): the norm
                                    # part that folds both into the next norm's launch, or `settle()`, applies it
         self.act = None        # h in the activations' storage type, where a block keeps such a copy beside it
+        self.lanes = None      # float32 [T, S, W]: S residual streams per token where a model keeps several (the
+                               # blocks of parts/block.py:HyperBlock); h is then stale until `close()`
+        self.pending_lanes = None   # (mix [S, S], out [S]): how `pending` enters the streams
+        self.closer = None     # what `close()` calls to bring h up to date from another form of the stream
 
     def settle(self) -> None:
         """Add a branch output that waits behind a norm of its own into the sum now."""
@@ -137,6 +141,13 @@ class ResidualStream:
             norm, delta = self.pending_norm, self.pending
             self.pending = self.pending_norm = None
             norm.add_normed(self, delta, None)
+
+    def close(self) -> None:
+        """Bring h up to date where blocks kept the stream in another form (several streams: their sum);
+        the model calls it before its final norm."""
+        if self.closer is not None:
+            closer, self.closer = self.closer, None
+            closer(self)
 
     def pending_tensor(self) -> Optional[torch.Tensor]:
         p = self.pending

@@ -6,6 +6,7 @@ from typing import Dict
 import torch
 
 from .. import ops
+from ..ops.profile import section
 from .base import LayerCache, ParamSpec, Part, ResidualStream, StepContext, TensorSource
 
 
@@ -140,3 +141,90 @@ class SandwichBlock(PreNormBlock):
             return
         n = self.norm2.after(self.norm1b, stream, y, ctx.act_dtype)
         stream.pending, stream.pending_norm = self.ffn.forward(n, ctx), self.norm2b
+
+
+class HyperConnection(Part):
+    """The weights by which one sublayer reads S residual streams and writes back into them: ``in`` [S]
+    (the sublayer's input is sum_s in[s] x_s), ``mix`` [S, S] indexed (from, to) and ``out`` [S] (every stream
+    at once, from the old ones: x_t <- sum_s mix[s, t] x_s + out[t] y).  Kept in float."""
+
+    def __init__(self, n_streams: int, names=None):
+        self.S = int(n_streams)
+        self.names = dict(names or {"in": "in", "out": "out", "mix": "mix"})
+        self.w_in = self.w_out = self.w_mix = None
+
+    def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
+        return {prefix + self.names["in"]: ParamSpec((self.S,)), prefix + self.names["out"]: ParamSpec((self.S,)),
+                prefix + self.names["mix"]: ParamSpec((self.S, self.S))}
+
+    def load(self, prefix: str, source: TensorSource) -> None:
+        self.w_in = source.get(prefix + self.names["in"]).float().contiguous()
+        self.w_out = source.get(prefix + self.names["out"]).float().contiguous()
+        self.w_mix = source.get(prefix + self.names["mix"]).float().contiguous()
+
+
+class HyperBlock(PreNormBlock):
+    """A pre-norm layer over S residual streams per token instead of one (hyper-connections): for each
+    sublayer (the mixer, then the feed-forward where there is one) u = sum_s in[s] x_s, y = sublayer(norm(u)),
+    and x_t <- sum_s mix[s, t] x_s + out[t] y for all streams at once.  The streams all start as the embedding
+    row, and the model's output reads their plain sum.
+
+    The streams live in ``stream.lanes`` (float32 [T, S, W]); a sublayer's output waits in ``stream.pending``
+    with its connection's weights (``stream.pending_lanes``) for the next launch of the one kernel
+    (csrc/hyper.hip) that brings the streams up to date, forms the next sublayer's input and normalises
+    it; the last output of the model is folded in where the streams are summed (``stream.close()``)."""
+
+    def __init__(self, n_streams: int, norm1: Part, mixer: Part, norm2: Part = None, ffn: Part = None, names=None):
+        super().__init__(norm1, mixer, norm2, ffn, names or {"norm1": "norm1", "mixer": "mix.", "norm2": "norm2", "ffn": "mlp.",
+                                                             "hc1": "hc1.", "hc2": "hc2."})
+        if not 1 <= n_streams <= ops.HYPER_MAX_STREAMS:
+            raise ValueError(f"{n_streams} residual streams are not taken: 1 to {ops.HYPER_MAX_STREAMS}")
+        self.S = int(n_streams)
+        self.hc1 = HyperConnection(self.S)
+        self.hc2 = HyperConnection(self.S) if ffn is not None else None
+
+    def _children(self):
+        kids = list(super()._children()) + [(self.names["hc1"], self.hc1)]
+        if self.hc2 is not None:
+            kids.append((self.names["hc2"], self.hc2))
+        return tuple(kids)
+
+    def _read(self, stream: ResidualStream, hc: HyperConnection, norm: Part, ctx: StepContext) -> torch.Tensor:
+        """The streams brought up to date with the output that waits, and the next sublayer's normalised input."""
+        T, W = stream.h.shape
+        if stream.lanes is None:
+            if stream.pending is not None or stream.pending_norm is not None:
+                raise ValueError("a block of several streams cannot follow one that leaves its output pending")
+            stream.lanes = torch.empty(T, self.S, W, dtype=torch.float32, device=stream.h.device)
+            src = stream.h                                   # every stream starts as this one row
+            stream.closer = _sum_of_lanes
+        else:
+            if stream.lanes.shape[1] != self.S:
+                raise ValueError("the layers of a model keep one number of residual streams")
+            src = stream.lanes
+        delta, mix, out_w = stream.pending, None, None
+        if delta is not None:
+            mix, out_w = stream.pending_lanes
+        with section("norm", nbytes=T * W * (8 * self.S + 4)):
+            n = ops.hyper_step(src, stream.lanes, self.S, delta, mix, out_w, hc.w_in, norm.weight, norm.eps, ctx.act_dtype)
+        stream.pending = stream.pending_lanes = None
+        return n
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: LayerCache) -> None:
+        n = self._read(stream, self.hc1, self.norm1, ctx)
+        stream.pending, stream.pending_lanes = self.mixer.forward(n, ctx, cache), (self.hc1.w_mix, self.hc1.w_out)
+        if self.ffn is not None:
+            n = self._read(stream, self.hc2, self.norm2, ctx)
+            stream.pending, stream.pending_lanes = self.ffn.forward(n, ctx), (self.hc2.w_mix, self.hc2.w_out)
+
+
+def _sum_of_lanes(stream: ResidualStream) -> None:
+    """h = the plain sum of the streams, the waiting output folded in first (the streams themselves are
+    not stored again: nobody reads them after this)."""
+    S = stream.lanes.shape[1]
+    delta, mix, out_w = stream.pending, None, None
+    if delta is not None:
+        mix, out_w = stream.pending_lanes
+    with section("norm", nbytes=stream.h.numel() * (4 * S + 4)):
+        stream.h = ops.hyper_step(stream.lanes, None, S, delta, mix, out_w)
+    stream.pending = stream.pending_lanes = stream.lanes = None

@@ -26,17 +26,18 @@ def _rows(w) -> torch.Tensor:
     return ops.unpack_weight(w) if isinstance(w, ops.PackedWeight) else w
 
 
-def _activation_code(name: str) -> int:
-    try:
-        return ops.ACTIVATIONS[name]
-    except KeyError:
-        raise ValueError(f"activation {name!r} is not known ({', '.join(sorted(ops.ACTIVATIONS))})") from None
+def _activation_code(name: str, limit: Optional[float] = None):
+    """What the kernels take for the gated unit `name` (a code, or a code with its limit)."""
+    if name not in ops.ACTIVATIONS:
+        raise ValueError(f"activation {name!r} is not known ({', '.join(sorted(ops.ACTIVATIONS))})")
+    return ops.gated_activation(name, limit)
 
 
 class DenseSwiGLU(Part):
     """down( act(gate x) * (up x) ) (reference: src/SharpInference.Engine/ForwardPass.cs:2006-2015;
     silu(g) = g / (1 + exp(-g)), src/SharpInference.Cpu/SimdKernels.cs:4377-4408).  ``activation``
-    names the gate's function: "silu" (the reference's) or "gelu_tanh".  ``bias``: the three
+    names the gate's function: "silu" (the reference's), "gelu_tanh", or "swish_clamp" with ``limit``:
+    g = min(gate x, limit), u = clamp(up x, -limit, limit), and the unit is g sigmoid(1.702 g) (u + 1).  ``bias``: the three
     products carry biases (``names`` + ``bias_suffix``), added in float: the gate's and the up
     projection's inside the activation kernel, the down projection's by a row kernel.  ``names``:
     the three matrices' names behind the part's prefix."""
@@ -44,9 +45,9 @@ class DenseSwiGLU(Part):
     NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
 
     def __init__(self, hidden: int, intermediate: int, activation: str = "silu", bias: bool = False,
-                 names: Optional[Dict[str, str]] = None, bias_suffix: str = ".bias"):
+                 names: Optional[Dict[str, str]] = None, bias_suffix: str = ".bias", limit: Optional[float] = None):
         self.hidden, self.inter = int(hidden), int(intermediate)
-        self.act = _activation_code(activation)
+        self.act = _activation_code(activation, limit)
         self.bias, self.bias_suffix = bool(bias), bias_suffix
         self.names = {**self.NAMES, **(names or {})}
         self.w_gate_up: Optional[torch.Tensor] = None
@@ -130,7 +131,10 @@ class MoESwiGLU(Part):
     order, src/SharpInference.Cuda/CudaKernels.cs:112-157 llm_moe_weighted_reduce).  The shared
     expert sees the unscaled input (2060-2066); the outputs are summed (2096-2097).  ``gate`` is "sigmoid" or "softmax"
     (2031-2034); ``renormalise`` divides the k scores by their sum (2156-2162); ``activation`` names the
-    experts' gate function ("silu", the reference's, or "gelu_tanh")."""
+    experts' gate function ("silu", the reference's, "gelu_tanh", or "swish_clamp" with ``limit``; the
+    shared expert may have a limit and a width of its own, ``shared_limit``).  ``gate`` "softmax_picked":
+    the largest logits are picked and their weights are the softmax over the picked logits alone.
+    ``router_bias``: a stored vector [E] is added to the router's logits."""
 
     MERGE_MAX_TOKENS = 16   # one row block of the few-rows kernel for the shared group (measured: up to 64 tokens
                             # the merged launches and the library's product for the shared expert are as fast)
@@ -139,12 +143,14 @@ class MoESwiGLU(Part):
                                    # the library's product for the shared expert (which runs at the matrix cores' peak)
 
     NAMES = {"router": "router.weight", "gate": "experts.gate_proj", "up": "experts.up_proj",
-             "down": "experts.down_proj", "shared": "shared_expert.", "correction": "router.correction"}
+             "down": "experts.down_proj", "shared": "shared_expert.", "correction": "router.correction",
+             "router_bias": "router.bias"}
 
     def __init__(self, hidden: int, num_experts: int, top_k: int, expert_intermediate: int,
                  shared_intermediate: Optional[int] = None, gate: str = "sigmoid", renormalise: bool = False,
                  score_on_input: bool = True, activation: str = "silu", correction: bool = False,
-                 n_groups: int = 1, keep_groups: int = 1, names: Optional[Dict[str, str]] = None):
+                 n_groups: int = 1, keep_groups: int = 1, names: Optional[Dict[str, str]] = None,
+                 limit: Optional[float] = None, shared_limit: Optional[float] = None, router_bias: bool = False):
         """``correction``: a stored vector [E] is added to the gate values where experts are chosen
         (the weights stay the gate values).  ``n_groups`` / ``keep_groups``: the experts form
         n_groups equal groups of neighbours and are chosen from the keep_groups best of them only
@@ -162,13 +168,17 @@ class MoESwiGLU(Part):
             raise ValueError(f"top_k {top_k} must lie in 1..{num_experts}")
         if num_experts > ops.ROUTER_MAX_EXPERTS:
             raise ValueError(f"{num_experts} experts are not taken: the routing kernels hold scores for {ops.ROUTER_MAX_EXPERTS}")
-        if gate not in ("sigmoid", "softmax"):
-            raise ValueError(f"router gate {gate!r} is not known (sigmoid, softmax)")
+        if gate not in ("sigmoid", "softmax", "softmax_picked"):
+            raise ValueError(f"router gate {gate!r} is not known (sigmoid, softmax, softmax_picked)")
         self.hidden, self.E, self.k = int(hidden), int(num_experts), int(top_k)
         self.inter = int(expert_intermediate)
-        self.act = _activation_code(activation)
-        self.shared = DenseSwiGLU(hidden, shared_intermediate, activation) if shared_intermediate else None
-        self.gate = ops.GATE_SIGMOID if gate == "sigmoid" else ops.GATE_SOFTMAX
+        self.act = _activation_code(activation, limit)
+        shared_names = {k: self.names[k] for k in ("shared_gate", "shared_up", "shared_down") if k in self.names}
+        self.shared = DenseSwiGLU(hidden, shared_intermediate, activation, limit=shared_limit if shared_limit is not None else limit,
+                                  names={k[len("shared_"):]: v for k, v in shared_names.items()} or None) if shared_intermediate else None
+        self.gate = {"sigmoid": ops.GATE_SIGMOID, "softmax": ops.GATE_SOFTMAX, "softmax_picked": ops.GATE_SOFTMAX_PICKED}[gate]
+        self.router_bias = bool(router_bias)
+        self.b_router: Optional[torch.Tensor] = None      # float32 [E]
         self.renormalise = bool(renormalise)
         self.score_on_input = bool(score_on_input)
         self.w_router: Optional[torch.Tensor] = None
@@ -199,17 +209,21 @@ class MoESwiGLU(Part):
         out.update(self._expert_specs(prefix, "down", (self.hidden, self.inter)))
         if self.correction:
             out[prefix + self.names["correction"]] = ParamSpec((self.E,))
+        if self.router_bias:
+            out[prefix + self.names["router_bias"]] = ParamSpec((self.E,))
         if self.shared is not None:
             out.update(self.shared.param_specs(prefix + self.names["shared"]))
         return out
 
     def _route_args(self) -> dict:
-        return dict(correction=self.w_correction, n_groups=self.n_groups, keep_groups=self.keep_groups)
+        return dict(correction=self.w_correction, n_groups=self.n_groups, keep_groups=self.keep_groups, bias=self.b_router)
 
     def load(self, prefix: str, source: TensorSource) -> None:
         self.w_router = source.get(prefix + self.names["router"])
         if self.correction:
             self.w_correction = source.get(prefix + self.names["correction"]).float().contiguous()
+        if self.router_bias:
+            self.b_router = source.get(prefix + self.names["router_bias"]).float().contiguous()
         g = self._expert_stack(prefix, "gate", source)
         u = self._expert_stack(prefix, "up", source)
         d = self._expert_stack(prefix, "down", source)
@@ -221,7 +235,7 @@ class MoESwiGLU(Part):
         # The experts' matrices are kept only in the order the kernels stream them (no rows: both
         # the few-rows and the many-rows product of the experts read that order), if the sizes allow.
         pack = bf16 and self.inter % 128 == 0 and self.hidden % 128 == 0
-        merge = (bf16 and sh is not None and sh.inter == self.inter and sh.w_gate_up.dtype == torch.bfloat16
+        merge = (bf16 and sh is not None and sh.inter == self.inter and sh.act == self.act and sh.w_gate_up.dtype == torch.bfloat16
                  and sh.w_down.dtype == torch.bfloat16)   # (dtype: of a tensor or of a packed weight)
         if not bf16:
             self.w_gate_up, self.w_down = _fuse_rows(g, u), d
@@ -291,7 +305,8 @@ class MoESwiGLU(Part):
         """The block's second half from the residual stream: normalise and feed forward.  With a
         few decode tokens the norm and the router are one launch (the bits of the two)."""
         T = stream.h.shape[0]
-        plain_choice = self.w_correction is None and self.keep_groups == self.n_groups   # what the fused kernel picks by
+        plain_choice = (self.w_correction is None and self.keep_groups == self.n_groups and self.b_router is None
+                        and self.gate != ops.GATE_SOFTMAX_PICKED)   # what the fused kernel picks by
         if (self._few_tokens(T, ctx) and isinstance(norm, RMSNorm) and plain_choice
                 and ops.norm_router_ok(stream.h, stream.pending, ctx.act_dtype)):
             with section("norm + router", nbytes=T * self.hidden * 10 + 2 * self.E * self.hidden):

@@ -1,5 +1,6 @@
 """Recurrent mixers whose state is a matrix per head with one scalar decay per token: a matrix memory
-with exponential gates, and a selective state space behind a short convolution."""
+with exponential gates, a selective state space behind a short convolution, and retention (a fixed
+decay per head)."""
 from __future__ import annotations
 
 from typing import Dict, Optional
@@ -219,4 +220,82 @@ class StateSpaceMixer(Part):
         with section("head norm + gate", nbytes=T * self.inner * (4 + 2 * width)):
             y = ops.group_norm_gate(y, self.w_norm, self.eps, self.norm_groups, ctx.act_dtype, proj, 0, ops.GATE_SILU, gate_first=True)
         with section("o", nbytes=width * self.hidden * (self.inner + T) + width * T * self.inner, flops=2.0 * T * self.hidden * self.inner):
+            return ops.linear(y, self.w_o, ctx.act_dtype)
+
+
+class Retention(Part):
+    """Retention: linear attention with one fixed decay per head, no softmax and no denominator.  With h the
+    input, per head (dk key channels, dv value channels): q = W_q h, k = W_k h, v = W_v h; q and k are turned
+    by rotary positions (``rotary``: pairs (i, i + r/2) of the leading r elements; None: no rotation), k is then
+    multiplied by dk^(-1/2); S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t; each head's output is divided by
+    its root mean square (no weight), the heads side by side are multiplied by silu(W_g h) and projected by W_o.
+
+    What is kept per request is S alone, in its state slot (``ops.walk_state_shape``): no pages.  The
+    rotation (on the staged floats, inside the walk), the state, its sums and the norm are float whatever
+    the activations are stored as.  A step walks each entry's tokens in order from the slot's state
+    (csrc/state_walk.hip), long entries in segments side by side."""
+
+    NAMES = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o"}
+
+    def __init__(self, hidden: int, num_heads: int, key_dim: int, value_dim: int, decays, norm_eps: float, rotary=None,
+                 names: Optional[Dict[str, str]] = None):
+        if min(num_heads, key_dim, value_dim) < 1:
+            raise ValueError("heads, key_dim and value_dim must be positive")
+        if key_dim > ops.WALK_MAX_KEY_DIM:
+            raise ValueError(f"{key_dim} key channels a head are not taken: at most {ops.WALK_MAX_KEY_DIM}")
+        decays = [float(d) for d in decays]
+        if len(decays) != num_heads or not all(0.0 < d <= 1.0 for d in decays):
+            raise ValueError("one decay in (0, 1] per head is wanted")
+        if rotary is not None and (rotary.pair_layout != "half" or rotary.head_dim != key_dim):
+            raise ValueError("retention turns split halves of its own key width")
+        self.hidden, self.nh, self.dk, self.dv = int(hidden), int(num_heads), int(key_dim), int(value_dim)
+        self.decays, self.eps, self.rotary = decays, float(norm_eps), rotary
+        self.names = {**self.NAMES, **(names or {})}
+        self.graph_safe = True         # entries and their state slots are read from the step's device arrays
+        self.w_in = None               # [q | k | v | g] rows: one product of the input
+        self.w_o = None
+        self._decay_t: Optional[torch.Tensor] = None
+
+    def step_planners(self):
+        return (WALK_SEGMENTS,)
+
+    def cache_spec(self) -> StateSpec:
+        return StateSpec(ops.walk_state_shape(self.nh, self.dk, self.dv, ops.WALK_FIXED_DECAY), torch.float32)
+
+    def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
+        n, qk, vv = self.names, self.nh * self.dk, self.nh * self.dv
+        return {
+            prefix + n["q"]: ParamSpec((qk, self.hidden)),
+            prefix + n["k"]: ParamSpec((qk, self.hidden)),
+            prefix + n["v"]: ParamSpec((vv, self.hidden)),
+            prefix + n["g"]: ParamSpec((vv, self.hidden)),
+            prefix + n["o"]: ParamSpec((self.hidden, vv)),
+        }
+
+    def load(self, prefix: str, source: TensorSource) -> None:
+        n = self.names
+        parts = [source.get(prefix + n[k]) for k in ("q", "k", "v", "g")]
+        self.w_in = ops.pack_weight(_fuse(parts, self.hidden))
+        self.w_o = ops.pack_weight(source.get(prefix + n["o"]))
+        self._decay_t = torch.tensor(self.decays, dtype=torch.float32, device=parts[0].device)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+        if not cache.write:
+            raise ValueError("a recurrent mixer's state cannot be shared between layers")
+        T = x.shape[0]
+        qk, vv = self.nh * self.dk, self.nh * self.dv
+        width = 2 if ctx.act_dtype == torch.bfloat16 else 4
+        n_in = 2 * qk + 2 * vv
+        with section("q|k|v|g", nbytes=width * n_in * (self.hidden + T) + width * T * self.hidden, flops=2.0 * T * self.hidden * n_in):
+            proj = ops.linear(x, self.w_in, ctx.act_dtype)
+        state = cache.states[0] if cache.states else cache.state
+        with section("recurrence", nbytes=lambda: 8 * ctx.n_entries * qk * self.dv + T * (width * (2 * qk + vv) + 4 * vv),
+                     flops=4.0 * T * qk * self.dv):
+            o = ops.state_walk(proj, 0, qk, 2 * qk, 1, None, (self._decay_t,), 0.0, 1.0, ops.WALK_FIXED_DECAY, state, ctx,
+                               self.nh, self.dk, self.dv, segments=_segments_for(ctx, self.nh, self.dv),
+                               inv_freq=self.rotary.table(x.device) if self.rotary is not None else None,
+                               k_scale=self.dk ** -0.5)
+        with section("head norm + gate", nbytes=T * vv * (4 + 2 * width)):
+            y = ops.group_norm_gate(o, None, self.eps, self.nh, ctx.act_dtype, proj, 2 * qk + vv, ops.GATE_SILU)
+        with section("o", nbytes=width * self.hidden * (vv + T) + width * T * vv, flops=2.0 * T * self.hidden * vv):
             return ops.linear(y, self.w_o, ctx.act_dtype)

@@ -61,4 +61,4 @@ def _ensure_builtin() -> None:
     if _builtin_done:
         return
     _builtin_done = True
-    from .models import kuvonex, llama4, nosedra, pazatar  # noqa: F401  (register themselves)
+    from .models import fovosun, kuvonex, llama4, nosedra, pazatar  # noqa: F401  (register themselves)
