@@ -294,3 +294,13 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int], store: Cal
         x = xs.sum(dim=0)
     hn = store(rms_norm(x, w["final.norm"], eps))
     return hn @ w["head"].T
+
+
+def generate(cfg: dict, w: Dict[str, torch.Tensor], prompt: List[int], n_new: int) -> List[int]:
+    """Greedy continuation: the whole sequence is recomputed for every new token."""
+    toks, out = list(prompt), []
+    for _ in range(n_new):
+        nxt = int(torch.argmax(forward(cfg, w, toks)[-1]))
+        toks.append(nxt)
+        out.append(nxt)
+    return out
