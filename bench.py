@@ -16,7 +16,9 @@ each beside Llama 4 layers of the same width, heads and experts, with the kernel
 ``--shape pazatar`` does the same for Pazatar layers (attention that norms before it rotates, gated linear
 attention beside it, dense feed-forwards) beside Llama 4 layers with dense feed-forwards;
 ``--shape nosedra`` runs Nosedra layers (attention with a learned sink beside a matrix memory with exponential
-gates, state-space layers) beside Pazatar layers of the same sizes.
+gates, state-space layers) beside Pazatar layers of the same sizes;
+``--shape fovosun`` runs Fovosun layers (differential attention, retention, clamped routed experts, four
+residual streams) beside Llama 4 layers of the same width, heads and experts.
 """
 from __future__ import annotations
 
@@ -658,6 +660,59 @@ def run_nosedra(args) -> int:
     return 0
 
 
+# ---------------------------------------------------------------------------
+# Fovosun beside Llama 4 at equal sizes
+# ---------------------------------------------------------------------------
+# width, layers (differential attention with a window, behind a convolution, retention, with a window again), heads
+# (two score maps of 64 over values of 128, where Llama 4 has heads of 128) in groups of 8 over a key head, retention
+# heads of 128 key and 128 value channels, routed experts, picks, expert width (and a shared expert of that width with
+# a limit of its own), four residual streams, vocabulary
+FOVOSUN_SIZES = {
+    "w2048": dict(width=2048, layers=4, heads=16, experts=64, top=6, ff=1408, vocab=32000, window=1024),
+    "w4096": dict(width=4096, layers=4, heads=32, experts=32, top=4, ff=2048, vocab=32000, window=1024),
+}
+FOVOSUN_KINDS = ["attention_2", "attention", "retention", "attention_2"]
+
+
+def fovosun_config(z: dict) -> dict:
+    kv = max(1, z["heads"] // 8)
+    windowed = {"heads": z["heads"], "kv_heads": kv, "dim": 64, "vdim": 128, "scale": 64 ** -0.5, "diff": 0.3,
+                "rot": {"base": 10000.0, "dims": 64}, "mask": {"size": z["window"]}}
+    conv = {"heads": z["heads"], "kv_heads": kv, "dim": 64, "vdim": 128, "scale": 64 ** -0.5, "diff": 0.3, "conv": 4,
+            "q_temp": {"coef": 0.1, "every": 1024}}
+    ret = {"heads": z["heads"], "dim": 128, "vdim": 128, "decay": [1.0 - 2.0 ** (-5 - 3 * h / z["heads"]) for h in range(z["heads"])],
+           "rot": {"base": 1000000.0, "dims": 64}}
+    mlp = {"kind": "moe", "expert": {"ff": z["ff"], "limit": 7.0}, "router": {"experts": z["experts"], "top": z["top"]},
+           "shared": {"ff": z["ff"], "limit": 3.0}}
+    mixers = {"attention_2": windowed, "attention": conv, "retention": ret}
+    layers = [{"type": kind, "mixer": mixers[kind], "mlp": mlp} for kind in FOVOSUN_KINDS[:z["layers"]]]
+    return {"architecture": "Fovosun", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+            "streams": 4, "layers": layers}
+
+
+def llama4_like_fovosun(z: dict) -> dict:
+    """Llama 4 layers of the same width, heads, kv heads, experts, picks and expert width, chunks of the window's size."""
+    cfg = llama4_config_like(z)
+    cfg.update({"attention_chunk_size": z["window"]})
+    return cfg
+
+
+def run_fovosun(args) -> int:
+    """Prefill of one 2,048-token prompt and decode at batch 8 and 64 for the Fovosun design at two sizes
+    (random weights), each beside Llama 4 layers of the same width, heads, experts and expert width, with the
+    per-kernel-class tables of one prefill and one decode step of both."""
+    rows, P, steps, warm = _beside(args, FOVOSUN_SIZES, (("fovosun", fovosun_config), ("llama4", llama4_like_fovosun)))
+    k0 = rows[0]
+    out = {"metric": "decode tok/s at batch 8 (Fovosun, width 2048, 4 layers, 2,048-token prompts)", "value": k0["decode_b8_tok_s"],
+           "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": k0["decode_b8_ms_per_step"],
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"model": "fovosun-random beside llama4-random at equal sizes", "global_batch": 8, "seq_len": CONTEXT,
+                      "parallelism": "single-gpu", "prompt_len": P, "sizes": FOVOSUN_SIZES},
+           "rows": rows}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -671,9 +726,10 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel instead of replaying a HIP graph")
     ap.add_argument("--no-peaks", action="store_true", help="skip the two measuring kernels (pure read, matrix-core loop)")
     ap.add_argument("--profile", action="store_true", help="also print ms / bytes / GB/s per kernel class of one prefill and one decode step")
-    ap.add_argument("--shape", default="scout", choices=["scout", "maverick8", "long16", "kuvonex", "pazatar", "nosedra"],
+    ap.add_argument("--shape", default="scout", choices=["scout", "maverick8", "long16", "kuvonex", "pazatar", "nosedra", "fovosun"],
                     help="scout: the headline run; maverick8 / long16: two other workloads; kuvonex / pazatar: that design beside "
-                         "Llama 4 layers of equal size; nosedra: that design beside Pazatar layers of equal size; each prints a JSON line of its own")
+                         "Llama 4 layers of equal size; nosedra: that design beside Pazatar layers of equal size; fovosun: that design beside "
+                         "Llama 4 layers of equal size; each prints a JSON line of its own")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path (N=1 only)")
@@ -688,6 +744,8 @@ def main() -> int:
         return run_pazatar(args)
     if args.shape == "nosedra":
         return run_nosedra(args)
+    if args.shape == "fovosun":
+        return run_fovosun(args)
 
     import torch  # noqa: F401
 

@@ -142,12 +142,14 @@ class ResidualStream:
             self.pending = self.pending_norm = None
             norm.add_normed(self, delta, None)
 
-    def close(self) -> None:
+    def close(self, rows: Optional[torch.Tensor] = None) -> bool:
         """Bring h up to date where blocks kept the stream in another form (several streams: their sum);
-        the model calls it before its final norm."""
-        if self.closer is not None:
-            closer, self.closer = self.closer, None
-            closer(self)
+        the model calls it before its final norm.  With ``rows`` (int32 token indices) a closer may leave
+        in h those rows alone, in that order: it then returns True."""
+        if self.closer is None:
+            return False
+        closer, self.closer = self.closer, None
+        return bool(closer(self, rows))
 
     def pending_tensor(self) -> Optional[torch.Tensor]:
         p = self.pending

@@ -218,13 +218,15 @@ class HyperBlock(PreNormBlock):
             stream.pending, stream.pending_lanes = self.ffn.forward(n, ctx), (self.hc2.w_mix, self.hc2.w_out)
 
 
-def _sum_of_lanes(stream: ResidualStream) -> None:
-    """h = the plain sum of the streams, the waiting output folded in first (the streams themselves are
-    not stored again: nobody reads them after this)."""
+def _sum_of_lanes(stream: ResidualStream, rows) -> bool:
+    """h = the plain sum of the streams, the waiting output folded in first, for the rows asked for
+    alone (the streams themselves are not stored again: nobody reads them after this)."""
     S = stream.lanes.shape[1]
     delta, mix, out_w = stream.pending, None, None
     if delta is not None:
         mix, out_w = stream.pending_lanes
-    with section("norm", nbytes=stream.h.numel() * (4 * S + 4)):
-        stream.h = ops.hyper_step(stream.lanes, None, S, delta, mix, out_w)
+    n = stream.h.shape[0] if rows is None else rows.shape[0]
+    with section("norm", nbytes=n * stream.h.shape[1] * (4 * S + 4)):
+        stream.h = ops.hyper_step(stream.lanes, None, S, delta, mix, out_w, rows=rows)
     stream.pending = stream.pending_lanes = stream.lanes = None
+    return rows is not None

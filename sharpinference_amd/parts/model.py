@@ -159,8 +159,8 @@ class DecoderModel(Part):
             self.blocks[r.layer].forward(stream, ctx, c)
         if logit_rows is None or logit_rows.numel() == 0:
             return None
-        stream.close()
-        n = self.final_norm.forward(stream, ctx.act_dtype, rows=logit_rows)
+        picked = stream.close(logit_rows)        # (several streams: their sum, for the wanted rows alone)
+        n = self.final_norm.forward(stream, ctx.act_dtype, rows=None if picked else logit_rows)
         m = n.shape[0]
         with section("head", nbytes=2 * self.vocab_size * self.hidden + 4 * m * self.vocab_size, flops=2.0 * m * self.vocab_size * self.hidden):
             logits = ops.linear(n, self.head, torch.float32)
