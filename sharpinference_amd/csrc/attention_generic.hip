@@ -12,7 +12,8 @@
 #include "common.h"
 
 constexpr int kAttnWaves = 4;
-constexpr int kAttnMaxHd = 256;
+constexpr int kAttnMaxHd = 256;      // widest value (a lane holds four output elements)
+constexpr int kAttnMaxKeyHd = 512;   // widest key (a head of two score maps side by side)
 
 template <typename T>
 __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
@@ -20,7 +21,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
     const int* __restrict__ block_table, const int* __restrict__ entry_of_token,
     const int* __restrict__ positions, T* __restrict__ out, int window_kind, int window, float scale, int nh,
     int nkv, int hd, int vd, int page_size, int max_blocks, int num_pages, float softcap, int sink, const float* __restrict__ sink_vals) {
-  __shared__ float qs[kAttnMaxHd];
+  __shared__ float qs[kAttnMaxKeyHd];
   __shared__ float pw[kAttnWaves][kWave];
   __shared__ int vrow[kAttnWaves][kWave];
   __shared__ float m_s[kAttnWaves], l_s[kAttnWaves];
@@ -132,7 +133,7 @@ SHARPI_EXPORT int sharpi_attention_generic(const void* q, const void* k_cache, c
                                            float scale, int n_tokens, int nh, int nkv, int hd, int vd, int page_size,
                                            int max_blocks, int num_pages, float softcap, int sink, const float* sink_vals, hipStream_t stream) {
   if (n_tokens <= 0) return SHARPI_OK;
-  if (hd <= 0 || hd > kAttnMaxHd || vd <= 0 || vd > kAttnMaxHd || nh <= 0 || nkv <= 0 || nh % nkv != 0 || nh > 65535) return SHARPI_ERR_ARG;
+  if (hd <= 0 || hd > kAttnMaxKeyHd || vd <= 0 || vd > kAttnMaxHd || nh <= 0 || nkv <= 0 || nh % nkv != 0 || nh > 65535) return SHARPI_ERR_ARG;
   if (page_size <= 0 || max_blocks <= 0 || num_pages <= 0) return SHARPI_ERR_ARG;
   if (window_kind < 0 || window_kind > 2 || (window_kind != 0 && window <= 0) || !(softcap >= 0.f)) return SHARPI_ERR_ARG;
   dim3 grid(n_tokens, nh), block(kAttnWaves * kWave);

@@ -56,11 +56,14 @@ struct PrepArgs {
   int temp_on;             // query temperature
   float temp_floor, temp_scale;
   int maps;                // score maps a head (1: the plain layout of q_out; > 1: q_out [T, nh * maps * hd], expanded)
+  int by8;                 // every offset, stride and width a multiple of 8 (and split halves): eight channels a thread
 };
+
+constexpr int kPrepMaxTurns = 256;    // rotary pairs whose cosines and sines a block keeps (a map of up to 512 elements)
 
 template <typename T>
 __global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
-  extern __shared__ float row[];          // q | k | v of the token, as floats
+  extern __shared__ __attribute__((aligned(32))) float row[];          // q | k | v of the token, as floats
   __shared__ float red[16];
   __shared__ float inv[kPrepMaxHeads];
   const int t = blockIdx.x;
@@ -83,7 +86,38 @@ __global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
   };
 
   // 1. gather, through the convolution where there is one
-  if (a.taps > 0) {
+  if (a.by8) {
+    // eight consecutive channels a thread, 16-byte loads (the sums of a channel are those of the scalar form)
+    const int e = a.taps > 0 ? a.entry_of_token[t] : 0;
+    const int li = a.taps > 0 ? t - a.cu_tokens[e] : 0;
+    const float* tail = a.taps > 0 ? a.tail + (size_t)a.state_slots[e] * (a.taps - 1) * C : nullptr;
+    for (int c = threadIdx.x * 8; c < C; c += kPrepThreads * 8) {
+      if (!mine(c)) continue;
+      const int col = c < qn ? a.q_off + c : c < qn + kn ? a.k_off + (c - qn) : a.v_off + (c - qn - kn);
+      float y[8];
+      if (a.taps > 0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = 0.f;
+        for (int j = 0; j < a.taps; ++j) {
+          const int back = a.taps - 1 - j;
+          float u[8];
+          if (back <= li) load8(proj + (size_t)(t - back) * a.stride + col, u);
+          else load8(tail + (size_t)(a.taps - 1 + li - back) * C + c, u);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) y[i] = fmaf(a.conv_w[(size_t)(c + i) * a.taps + j], u[i], y[i]);
+        }
+      } else {
+        load8(proj + (size_t)t * a.stride + col, y);
+        if (a.bias) {
+          float b8[8];
+          load8(a.bias + c, b8);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) y[i] += b8[i];
+        }
+      }
+      store8(row + c, y);
+    }
+  } else if (a.taps > 0) {
     const int e = a.entry_of_token[t];
     const int li = t - a.cu_tokens[e];                 // the token's place in its entry
     const float* tail = a.tail + (size_t)a.state_slots[e] * (a.taps - 1) * C;
@@ -147,11 +181,81 @@ __global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
 
   // 4. norm, rotation, and out: a thread takes a pair of a head (or two elements that do not turn)
   const float pos = (float)a.positions[t];
+  __shared__ float cs_tab[kPrepMaxTurns], sn_tab[kPrepMaxTurns];      // the token's angles are the same for every head and map
+  if (a.inv_freq) {
+    for (int i = threadIdx.x; i < a.rotary_dim / 2; i += kPrepThreads) {
+      const float ang = pos * a.inv_freq[i];
+      cs_tab[i] = cosf(ang) * a.magnitude;
+      sn_tab[i] = sinf(ang) * a.magnitude;
+    }
+    __syncthreads();
+  }
   const int sd = a.hd / a.maps;                          // width of one map of a head (the head's, with one map)
   const int half_hd = a.hd / 2, half_sd = sd / 2, half_r = a.rotary_dim / 2;
   T* qo = (T*)a.q_out + (size_t)t * qn * a.maps;
   T* kc = (T*)a.k_cache;
   const float temp = a.temp_on ? 1.0f + a.temp_scale * logf(floorf((pos + 1.0f) / a.temp_floor) + 1.0f) : 1.0f;
+  if (a.by8) {
+    // Eight consecutive elements a thread, 16-byte stores.  A run in the low half of a map's rotated part comes
+    // with its partner run half the rotated width on (the thread turns both); a run behind the rotated part passes.
+    const int runs = sd / 8, low = half_r / 8, rot_runs = a.rotary_dim / 8;
+    const int per_map = runs - low;                      // work items of a map: low runs (each with its partner) and the rest
+    const int page = slot >= 0 ? slot / a.page_size : 0, off = slot >= 0 ? slot % a.page_size : 0;
+    for (int i = threadIdx.x; i < heads * a.maps * per_map; i += kPrepThreads) {
+      const int hs = i / per_map, wi = i % per_map;
+      const int h = hs / a.maps, mp = hs % a.maps, at = mp * sd;
+      if (!all && !(h < a.nh ? (h >= qh0 && h < qh1) : (h - a.nh >= kh0 && h - a.nh < kh1))) continue;
+      const bool is_q = h < a.nh, turns = wi < low;
+      if (!is_q && slot < 0) continue;
+      const int e0 = at + (turns ? wi * 8 : (rot_runs + (wi - low)) * 8);      // first element inside the head
+      const int e1 = e0 + half_r;                                               // the partner run (turning runs only)
+      float x0[8], x1[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      load8(row + (size_t)h * a.hd + e0, x0);
+      if (turns) load8(row + (size_t)h * a.hd + e1, x1);
+      if (a.norm_mode != NORM_NONE) {
+        const float* w = is_q ? a.q_norm_w : a.k_norm_w;
+        const int wbase = a.norm_mode == NORM_WHOLE ? (is_q ? h : h - a.nh) * a.hd : 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          x0[j] = x0[j] * inv[h] * w[wbase + e0 + j];
+          if (turns) x1[j] = x1[j] * inv[h] * w[wbase + e1 + j];
+        }
+      }
+      if (turns) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float c = cs_tab[wi * 8 + j], sn = sn_tab[wi * 8 + j];
+          const float y0 = x0[j] * c - x1[j] * sn, y1 = x1[j] * c + x0[j] * sn;
+          x0[j] = y0;
+          x1[j] = y1;
+        }
+      }
+      if (is_q) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          x0[j] *= temp;
+          x1[j] *= temp;
+        }
+        if (a.maps == 1) {
+          store8(qo + (size_t)h * a.hd + e0, x0);
+          if (turns) store8(qo + (size_t)h * a.hd + e1, x1);
+        } else {
+          const float zero[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          T* qr = qo + ((size_t)h * a.maps + mp) * a.hd;
+          for (int mm = 0; mm < a.maps; ++mm) {
+            const int sh = (mm - mp) * sd;
+            store8(qr + e0 + sh, mm == mp ? x0 : zero);
+            if (turns) store8(qr + e1 + sh, mm == mp ? x1 : zero);
+          }
+        }
+      } else {
+        T* kr = kc + (((size_t)page * a.nkv + (h - a.nh)) * a.page_size + off) * a.hd;
+        store8(kr + e0, x0);
+        if (turns) store8(kr + e1, x1);
+      }
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < heads * half_hd; i += kPrepThreads) {
     const int hs = i / half_sd, pi = i % half_sd;         // (head, map) and the pair inside the map
     const int h = hs / a.maps, mp = hs % a.maps, at = mp * sd;
@@ -178,8 +282,7 @@ __global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
       x1 = x1 * inv[h] * w[wbase + d1];
     }
     if (turns && a.inv_freq) {
-      const float ang = pos * a.inv_freq[pi];
-      const float c = cosf(ang) * a.magnitude, s = sinf(ang) * a.magnitude;
+      const float c = cs_tab[pi], s = sn_tab[pi];
       const float y0 = x0 * c - x1 * s, y1 = x1 * c + x0 * s;
       x0 = y0;
       x1 = y1;
@@ -260,10 +363,16 @@ SHARPI_EXPORT int sharpi_qk_prep(const void* proj, int dtype, int stride, int q_
   const size_t lds = (size_t)(qn + kn + vn) * sizeof(float);
   if (lds > 60 * 1024) return SHARPI_ERR_ARG;
   const int parts = (n_tokens <= kPrepSplitTokens && nkv > 1 && nkv <= 65535 && nh % nkv == 0) ? nkv : 1;
+  auto at16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 32 == 0; };
+  const int sd = hd / maps;
+  const int by8 = (half_split || rotary_dim == 0) && rotary_dim % 16 == 0 && sd % 8 == 0 && vd % 8 == 0 &&
+                  stride % 8 == 0 && q_off % 8 == 0 && k_off % 8 == 0 && (v_off < 0 || v_off % 8 == 0) && at16(proj) && at16(q_out) &&
+                  at16(k_cache) && at16(tail) && at16(bias) && rotary_dim / 2 <= kPrepMaxTurns;
+  if (rotary_dim / 2 > kPrepMaxTurns) return SHARPI_ERR_ARG;
   PrepArgs a{proj, stride, q_off, k_off, v_off, nh, nkv, hd, vd, conv_w, taps, tail, state_slots, entry_of_token,
              cu_tokens, positions, norm_mode, q_norm_w, k_norm_w, eps, rotary_dim > 0 ? inv_freq : nullptr, rotary_dim,
              half_split, magnitude, q_out, k_cache, v_cache, slot_mapping, page_size, parts, bias, temp_on, temp_floor,
-             temp_scale, maps};
+             temp_scale, maps, by8};
   dim3 pgrid(n_tokens, parts);
   if (dtype == DT_F32) qk_prep_kernel<float><<<pgrid, kPrepThreads, lds, stream>>>(a);
   else if (dtype == DT_BF16) qk_prep_kernel<bf16_t><<<pgrid, kPrepThreads, lds, stream>>>(a);

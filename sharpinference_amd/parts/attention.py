@@ -123,8 +123,9 @@ class Attention(Part):
         if rotary is not None and rotary.head_dim != head_dim:
             raise ValueError("the rotary table's head_dim differs from the mixer's")
         head_dim = int(head_dim) * self.maps              # a head as the cache and the kernels see it: its maps side by side
-        if head_dim % 2 or not 2 <= head_dim <= 256:      # (the rotation takes pairs; the attention kernels hold 256 elements)
-            raise ValueError(f"head_dim {head_dim} is not taken: even sizes from 2 to 256")
+        widest = 256 * self.maps                          # (the rotation takes pairs; the attention kernels hold 256 elements a map)
+        if head_dim % 2 or not 2 <= head_dim <= widest:
+            raise ValueError(f"head_dim {head_dim} is not taken: even sizes from 2 to {widest}")
         if rotary is not None and rotary.pair_layout not in ("interleaved", "half"):
             raise ValueError(f"pair layout {rotary.pair_layout!r} is not taken by the rotation kernel")
         self.hidden, self.nh, self.nkv, self.hd = int(hidden), int(num_heads), int(num_kv_heads), int(head_dim)

@@ -77,11 +77,11 @@ WIDE = {
     ],
 }
 
-# one stream kept the way several are
+# one stream kept the way several are; score maps of 136 elements (a head's two maps are wider than any value row)
 ONE = {
     "architecture": "Fovosun", "vocab": 50, "width": 64, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.5}, "streams": 1,
     "layers": [
-        _layer(_diff("attention", 2, 1, 16, 32, 0.3, 0.2, q_temp=(0.5, 8)), _dense(32, 1.0)),
+        _layer(_diff("attention", 2, 1, 136, 32, 0.09, 0.2, q_temp=(0.5, 8)), _dense(32, 1.0)),
         _layer(_ret(2, 16, 8, (0.9, 0.99), rot=(100.0, 16)), _moe(4, 2, 16, 1.0)),
     ],
 }
